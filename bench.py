@@ -1,0 +1,184 @@
+"""Benchmark of the padding-free BERT encoder on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--no-cpu]
+
+A step is one pass Input -> L x Layer -> Output over one synthetic batch that is already
+resident in HBM.  Prints ONE JSON line: valid tokens/s (whole job), ms/step, the roofline of the
+dominant kernel measured live with HIP events, per-kernel rooflines, and the CPU baseline (the
+standard padded BERT encoder graph on the host cores, on a bounded sample of the same batch).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"fp16": 2500.0, "fp32": 157.3}
+
+
+def _time_kernel(fn, iters, warm=3):
+    import torch
+    for _ in range(warm):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters          # ms per launch
+
+
+def per_kernel(wl, T, mask_np, iters=20):
+    """Times every kernel of the path in isolation at the workload's real shapes and prices it
+    against its roofline with ALGORITHMIC bytes / flops."""
+    import numpy as np
+    import torch
+    from effective_transformer_amd import kernel_ops as k, ops
+
+    dt = torch.float16 if wl.dtype == "fp16" else torch.float32
+    e = 2 if wl.dtype == "fp16" else 4
+    B, S, H, F, heads, d = wl.B, wl.S, wl.H, wl.F, wl.heads, wl.d
+    g = torch.Generator(device="cuda").manual_seed(0)
+    rnd = lambda *s: torch.randn(*s, device="cuda", dtype=torch.float32, generator=g).to(dt)
+    x = rnd(B, S, H)
+    mask = torch.from_numpy(mask_np).cuda()
+    attr = mask[:, None, :].expand(B, S, S).to(dt).contiguous()
+    to, vwn, bidx, widx = ops.effective_transformer_input(x, mask, B, S, S, heads, d)
+    res = {}
+
+    def add(name, ms, bound, work):
+        if bound == "hbm":
+            ach, peak, unit = work / ms / 1e6, HBM_PEAK_GBS, "GB/s"
+        else:
+            ach, peak, unit = work / ms / 1e9, MFMA_PEAK_TFLOPS[wl.dtype], "TFLOP/s"
+        res[name] = {"ms": round(ms, 5), "bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": unit,
+                     "frac": round(ach / peak, 4)}
+
+    # input op = scan + index build + compress; output op = restore
+    ms = _time_kernel(lambda: ops.effective_transformer_input(x, mask, B, S, S, heads, d), iters)
+    add("input_scan_compress", ms, "hbm", 2 * T * H * e + 4 * B * S + 8 * T + 4)
+    ms = _time_kernel(lambda: ops.effective_transformer_output(to, vwn, bidx, widx, B, S, S, heads, d), iters)
+    add("output_restore", ms, "hbm", T * H * e + B * S * H * e + 8 * T)
+    # row kernels
+    a = rnd(T, H); r = rnd(T, H); bias = rnd(H); gam = rnd(H); bet = rnd(H)
+    ms = _time_kernel(lambda: k.add_bias_input_layernorm(a, r, bias, gam, bet), iters)
+    add("bias_residual_layernorm", ms, "hbm", 3 * T * H * e + 3 * H * e)
+    inter = rnd(T, F) * 0.1; bF = rnd(F)
+    ms = _time_kernel(lambda: k.add_bias_act(inter, bF), iters)
+    add("bias_gelu", ms, "hbm", 2 * T * F * e + F * e)
+    # fused attention on packed rows
+    qkv = rnd(B * S, 3 * H)
+    ctx = torch.empty(B * S, H, device="cuda", dtype=dt)
+    ms = _time_kernel(lambda: k.attention(qkv, qkv[:, H:], qkv[:, 2 * H:], 1, 3 * H, attr, vwn, B, S, heads, d, bidx,
+                                          widx, dst=ctx), iters)
+    lens = mask_np.sum(axis=1).astype(np.float64)
+    add("attention", ms, "hbm", 4 * T * H * e + B * S * S * e + 8 * T)
+    res["attention"]["valid_tflops"] = round(4 * H * float((lens ** 2).sum()) / ms / 1e9, 2)
+    # the four projections
+    for name, n, kk in (("gemm_qkv", 3 * H, H), ("gemm_attn_out", H, H), ("gemm_ffn_up", F, H), ("gemm_ffn_down", H, F)):
+        A = rnd(T, kk); Bm = rnd(kk, n) * 0.02
+        Cm = torch.empty(T, n, device="cuda", dtype=dt)
+        ms = _time_kernel(lambda: k.gemm(A, Bm, out=Cm), iters)
+        add(name, ms, "mfma", 2.0 * T * n * kk)
+    return res
+
+
+def cpu_baseline(w, nseq):
+    """The standard padded BERT encoder graph (the reference's comparison path) in fp32 on the host
+    cores, on the first `nseq` sequences of the batch, all layers."""
+    import numpy as np
+    import torch
+    from oracle import et_oracle as o
+    wl = w["wl"]
+    x = w["x"][:nseq].astype(np.float32)
+    attr = w["attr_mask"][:nseq].astype(np.float32)
+    weights = [a.astype(np.float32) for a in w["weights"]]
+    o.tf_graph_encoder(x[:4], attr[:4], weights[:16], wl.heads, wl.d)          # warm-up
+    t0 = time.perf_counter()
+    o.tf_graph_encoder(x, attr, weights, wl.heads, wl.d)
+    dtm = time.perf_counter() - t0
+    tokens = int(w["mask"][:nseq].sum())
+    return {"value": round(tokens / dtm, 1), "unit": "valid tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_batch_extrapolated": round(dtm * 1e3 * wl.B / nseq, 1),
+            "sample": "first %d of %d sequences (%d valid tokens), all %d layers, fp32, padded [B*S,H] graph"
+                      % (nseq, wl.B, tokens, wl.layers)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)       # the reference's 128 timed iterations
+    ap.add_argument("--warmup", type=int, default=10)       # ... after 10 warm-ups
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--cpu-seqs", type=int, default=0)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every box here has one); --gpus %d is not supported" % a.gpus)
+
+    import numpy as np
+    import torch
+    from effective_transformer_amd import _lib, ops
+    from oracle import et_oracle as o
+
+    _lib.load()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    w = o.make_workload(a.workload)
+    wl = w["wl"]
+    dt = torch.float16 if wl.dtype == "fp16" else torch.float32
+    enc = ops.EffectiveTransformerEncoder(wl.layers, wl.heads, wl.d, w["weights"], dt, "cuda:0")
+    x = torch.from_numpy(w["x"]).cuda()
+    mask = torch.from_numpy(w["mask"]).cuda()
+    attr = torch.from_numpy(w["attr_mask"]).cuda()
+    T = int(w["mask"].sum())
+
+    for _ in range(a.warmup):
+        enc(x, mask, attr)
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    s.record()
+    for _ in range(a.steps):
+        out = enc(x, mask, attr)
+    e.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    ms = s.elapsed_time(e) / a.steps
+
+    kernels = {} if a.no_kernels else per_kernel(wl, T, w["mask"])
+    roof = None
+    if kernels:
+        # dominant kernel = the largest share of a layer's time
+        share = {n: v["ms"] for n, v in kernels.items() if n.startswith("gemm") or n in ("attention", "bias_gelu")}
+        share["bias_residual_layernorm"] = 2 * kernels["bias_residual_layernorm"]["ms"]
+        dom = max(share, key=share.get)
+        kd = kernels[dom]
+        roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved"], "peak": kd["peak"], "unit": kd["unit"],
+                "frac": kd["frac"], "traffic": None}
+    cpu = None
+    if not a.no_cpu:
+        cpu = cpu_baseline(w, a.cpu_seqs or max(4, min(wl.B, 100 if wl.S <= 64 else 32)))
+
+    print(json.dumps({
+        "metric": "valid_tokens_per_s", "value": round(T / (ms / 1e3), 1), "unit": "valid tokens/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
+        "wall_ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": wl.dtype, "data": "synthetic",
+        "config": {"workload": "%s: BERT %d layers, hidden %d, %d heads x %d, FFN %d, batch %d, max_seq %d, %d valid tokens"
+                               % (wl.name, wl.layers, wl.H, wl.heads, wl.d, wl.F, wl.B, wl.S, T),
+                   "valid_tokens": T, "padded_tokens": wl.B * wl.S},
+        "roofline": roof, "kernels": kernels, "cpu_baseline": cpu,
+    }))
+
+
+if __name__ == "__main__":
+    main()

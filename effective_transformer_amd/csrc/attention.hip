@@ -1,0 +1,506 @@
+// Attention side of the encoder layer on gfx950.
+//   qkv_bias_pad      : [T,H] + bias -> zero-padded [B,heads,S,d]   (reference: cuda/attention.cu:105-242,
+//                                                                    zero fill tf_op/bert_transformer_op.cu.cc:146)
+//   softmax           : masked, scaled softmax in place             (cuda/attention.cu:249-382)
+//   transpose_rm_pad  : [B,heads,S,d] -> packed [T,H]               (cuda/attention.cu:387-492)
+//   attention (fused) : QK^T, masked softmax, PV and un-padding in one kernel
+//                       (tf_op/bert_transformer_op.cu.cc:159-192); reads Q/K/V either from the padded
+//                       buffers or straight from packed token rows, writes packed [T,H].
+//
+// Softmax semantics (both kernels): t = qk*scale + (1-mask)*(-10000); m = max(max_k t, 0);
+// e = exp(t-m); p = e / (sum e + 1e-6).  In fp16 the score is rounded to half before the softmax
+// and the probability after it, as the reference stores both in half.
+#include "et_device.hpp"
+#include "kernels.hpp"
+
+namespace et {
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T> struct Chunk16;
+template <> struct Chunk16<float> {
+  float4v v;
+  static constexpr int kElems = 4;
+};
+template <> struct Chunk16<_Float16> {
+  half8 v;
+  static constexpr int kElems = 8;
+};
+
+// ------------------------------------------------------------------------------------------
+// add bias + head split + re-pad, one workgroup per (sequence, matrix).  Every 16-byte chunk of
+// the padded destination is written once: bias-added data where a token exists, zero elsewhere.
+// ------------------------------------------------------------------------------------------
+constexpr int kPadThreads = 256;
+constexpr int kPadMaxSeq = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(kPadThreads) void qkv_bias_pad_kernel(
+    const T* __restrict__ Q, const T* __restrict__ bQ, const T* __restrict__ K, const T* __restrict__ bK,
+    const T* __restrict__ V, const T* __restrict__ bV, T* __restrict__ q_buf, T* __restrict__ k_buf,
+    T* __restrict__ v_buf, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ word_idx, int seq_len,
+    int heads, int d) {
+  using C = Chunk16<T>;
+  __shared__ int tok_of_pos[kPadMaxSeq];
+  const int b = blockIdx.x;
+  const int mat = blockIdx.y;
+  const T* src = mat == 0 ? Q : (mat == 1 ? K : V);
+  const T* bias = mat == 0 ? bQ : (mat == 1 ? bK : bV);
+  T* dst = mat == 0 ? q_buf : (mat == 1 ? k_buf : v_buf);
+  for (int s = threadIdx.x; s < seq_len; s += kPadThreads) tok_of_pos[s] = -1;
+  __syncthreads();
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  for (int t = t0 + threadIdx.x; t < t1; t += kPadThreads) {
+    const int s = word_idx[t];
+    if (s >= 0 && s < seq_len) tok_of_pos[s] = t;
+  }
+  __syncthreads();
+  const int cpd = d / C::kElems;           // chunks per head row
+  const int cph = heads * cpd;             // chunks per token row
+  const int total = heads * seq_len * cpd;
+  C* out = reinterpret_cast<C*>(dst) + (size_t)b * total;
+  const C* in = reinterpret_cast<const C*>(src);
+  const C* bi = reinterpret_cast<const C*>(bias);
+  for (int i = threadIdx.x; i < total; i += kPadThreads) {
+    const int c = i % cpd;
+    const int s = (i / cpd) % seq_len;
+    const int head = i / (cpd * seq_len);
+    const int t = tok_of_pos[s];
+    C val;
+    if (t >= 0) {
+      val.v = in[(size_t)t * cph + head * cpd + c].v + bi[head * cpd + c].v;
+    } else {
+#pragma unroll
+      for (int j = 0; j < C::kElems; ++j) val.v[j] = (T)0;
+    }
+    out[i] = val;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// stand-alone softmax: one wavefront per (b, head, q) row, up to 512 keys.
+// ------------------------------------------------------------------------------------------
+constexpr int kSmThreads = 256;
+constexpr int kSmMaxIters = 8;
+
+template <typename T>
+__global__ __launch_bounds__(kSmThreads) void softmax_kernel(T* __restrict__ qk, const T* __restrict__ attr_mask,
+                                                             int rows_total, int heads, int seq_len, float scaler) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = blockIdx.x * (kSmThreads / kWave) + threadIdx.x / kWave;
+  if (row >= rows_total) return;          // wave-uniform
+  const int q = row % seq_len;
+  const int b = row / (seq_len * heads);
+  T* x = qk + (size_t)row * seq_len;
+  const T* mk = attr_mask + ((size_t)b * seq_len + q) * seq_len;
+  float t[kSmMaxIters];
+  float mx = 0.f;                         // the maximum is clamped below at 0
+#pragma unroll
+  for (int i = 0; i < kSmMaxIters; ++i) {
+    const int k = lane + i * kWave;
+    t[i] = -INFINITY;
+    if (k < seq_len) {
+      t[i] = (float)x[k] * scaler + (1.0f - (float)mk[k]) * -10000.0f;
+      mx = fmaxf(mx, t[i]);
+    }
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kSmMaxIters; ++i) {
+    t[i] = __builtin_amdgcn_exp2f((t[i] - mx) * kLog2e);   // exp2(-inf) = 0 for absent keys
+    sum += t[i];
+  }
+  sum = wave_sum(sum) + 1e-6f;
+#pragma unroll
+  for (int i = 0; i < kSmMaxIters; ++i) {
+    const int k = lane + i * kWave;
+    if (k < seq_len) x[k] = (T)(t[i] / sum);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// un-pad + head merge: gather flattened over (packed row, 16-byte chunk).
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_rm_padding_kernel(
+    const T* __restrict__ src, T* __restrict__ dst, const int32_t* __restrict__ rows_dev, int rows_bound, int seq_len,
+    int heads, int cpd, const int32_t* __restrict__ batch_idx, const int32_t* __restrict__ word_idx) {
+  using C = Chunk16<T>;
+  const int rows = rows_dev ? min(*rows_dev, rows_bound) : rows_bound;
+  const int cph = heads * cpd;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long)rows * cph) return;
+  const int t = (int)(i / cph);
+  const int c = (int)(i - (long)t * cph);
+  const int head = c / cpd;
+  const int cc = c - head * cpd;
+  const int b = batch_idx[t], s = word_idx[t];
+  reinterpret_cast<C*>(dst)[i] =
+      reinterpret_cast<const C*>(src)[(((size_t)b * heads + head) * seq_len + s) * cpd + cc];
+}
+
+// ------------------------------------------------------------------------------------------
+// fused attention, size_per_head = 64, seq_len <= 128.
+//
+// One workgroup (4 wavefronts) per (sequence, head).  The sequence's K rows and the transpose of
+// its V rows are staged in LDS at their padded positions (zero where no token exists, so that a
+// mask that attends to a padded key sees the zero score / zero value the reference's padded
+// buffers hold); Q rows are staged beside them.  Each wavefront takes 16-query tiles:
+//   S^T = K Q^T   on v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x4_f32 -> a lane owns one query
+//                 column and 4 keys of every 16-key tile,
+//   softmax       over the lane's values + 2 cross-lane steps (lanes l, l^16, l^32, l^48 share a query),
+//   O^T = V^T P^T where the lane's own probability registers already are the B operand,
+//   then the lane writes 4 consecutive features of its query's packed output row.
+// Key tiles that hold no token skip their MFMAs (score 0, value 0) but still go through the
+// masked softmax, so the result equals the padded computation exactly.
+// ------------------------------------------------------------------------------------------
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kD = 64;
+
+template <typename T> struct AttnCfg;
+template <> struct AttnCfg<_Float16> {
+  static constexpr int kQkStride = kD + 8;   // halves; 144-byte rows keep 16-byte reads of 8 consecutive rows on distinct banks
+  static constexpr int kVtPad = 4;           // halves
+};
+template <> struct AttnCfg<float> {
+  static constexpr int kQkStride = kD + 4;   // floats; 272-byte rows
+  static constexpr int kVtPad = 4;           // floats
+};
+
+template <typename T, int NKT>
+struct AttnSmem {
+  static constexpr int kSp = NKT * 16;
+  static constexpr int kVtStride = kSp + AttnCfg<T>::kVtPad;
+  static constexpr size_t kQBytes = (size_t)kSp * AttnCfg<T>::kQkStride * sizeof(T);
+  static constexpr size_t kVtBytes = (size_t)kD * kVtStride * sizeof(T);
+  static constexpr size_t kBytes = 2 * kQBytes + kVtBytes + kSp * sizeof(int);
+};
+
+__device__ __forceinline__ float xor_lanes_16_32_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  v = fmaxf(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+__device__ __forceinline__ float xor_lanes_16_32_sum(float v) {
+  v += __shfl_xor(v, 16, kWave);
+  v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+template <typename T, int NKT>
+__global__ __launch_bounds__(kAttnThreads) void attention_kernel(
+    const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
+    const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ word_idx, int seq_len, int heads, float scaler) {
+  using Cfg = AttnCfg<T>;
+  using Sm = AttnSmem<T, NKT>;
+  using C = Chunk16<T>;
+  constexpr int kQS = Cfg::kQkStride;
+  constexpr int kVS = Sm::kVtStride;
+  constexpr int kSp = Sm::kSp;
+  constexpr int kCpr = kD / C::kElems;       // 16-byte chunks per head row
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* Qs = reinterpret_cast<T*>(smem_raw);
+  T* Ks = reinterpret_cast<T*>(smem_raw + Sm::kQBytes);
+  T* Vt = reinterpret_cast<T*>(smem_raw + 2 * Sm::kQBytes);
+  int* tok_of_pos = reinterpret_cast<int*>(smem_raw + 2 * Sm::kQBytes + Sm::kVtBytes);
+
+  const int head = blockIdx.x;
+  const int b = blockIdx.y;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  const int len = t1 - t0;
+  if (len <= 0) return;
+  const int H = heads * kD;
+  // positions are ascending inside a sequence: the last token bounds the occupied tiles
+  const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
+  const int n_tiles = last_pos / 16 + 1;    // 16-row tiles that hold at least one token (queries and keys)
+
+  // ---- stage: zero the key/value tiles in use, then scatter the sequence's rows --------------
+  for (int i = threadIdx.x; i < kSp; i += kAttnThreads) tok_of_pos[i] = -1;
+  {
+    const int rows = n_tiles * 16;
+    uint32_t* kz = reinterpret_cast<uint32_t*>(Ks);
+    const int kwords = rows * kQS * (int)sizeof(T) / 4;
+    for (int i = threadIdx.x; i < kwords; i += kAttnThreads) kz[i] = 0u;
+    uint32_t* vz = reinterpret_cast<uint32_t*>(Vt);
+    const int vwords = kD * kVS * (int)sizeof(T) / 4;
+    for (int i = threadIdx.x; i < vwords; i += kAttnThreads) vz[i] = 0u;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < len * kCpr; i += kAttnThreads) {
+    const int tt = i / kCpr;
+    const int c = i - tt * kCpr;
+    const int t = t0 + tt;
+    const int pos = word_idx[t];
+    if (pos < 0 || pos >= seq_len) continue;
+    size_t off;
+    if (layout == 1) {
+      off = (size_t)t * packed_ld + head * kD + c * C::kElems;
+    } else {
+      off = (((size_t)b * heads + head) * seq_len + pos) * kD + c * C::kElems;
+    }
+    const C qv = *reinterpret_cast<const C*>(q_src + off);
+    const C kv = *reinterpret_cast<const C*>(k_src + off);
+    const C vv = *reinterpret_cast<const C*>(v_src + off);
+    *reinterpret_cast<C*>(Qs + pos * kQS + c * C::kElems) = qv;
+    *reinterpret_cast<C*>(Ks + pos * kQS + c * C::kElems) = kv;
+#pragma unroll
+    for (int j = 0; j < C::kElems; ++j) Vt[(c * C::kElems + j) * kVS + pos] = vv.v[j];
+    if (c == 0) tok_of_pos[pos] = t;
+  }
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int l16 = lane & 15;
+  const int g = lane >> 4;
+
+  for (int qt = wave; qt < n_tiles; qt += kAttnWaves) {
+    const int q = qt * 16 + l16;            // this lane's query position
+    float s[NKT][4];
+    // ---- S^T = K Q^T -------------------------------------------------------------------
+    if constexpr (sizeof(T) == 2) {
+      half8 bq[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) bq[ks] = *reinterpret_cast<const half8*>(Qs + q * kQS + ks * 32 + g * 8);
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        float4v acc = {0.f, 0.f, 0.f, 0.f};
+        if (kt < n_tiles) {
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks) {
+            const half8 a = *reinterpret_cast<const half8*>(Ks + (kt * 16 + l16) * kQS + ks * 32 + g * 8);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bq[ks], acc, 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] = h2f(f2h(acc[r]));   // the score is stored in half
+      }
+    } else {
+      float bq[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4v v4 = *reinterpret_cast<const float4v*>(Qs + q * kQS + g * 16 + i * 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bq[i * 4 + j] = v4[j];
+      }
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        float4v acc = {0.f, 0.f, 0.f, 0.f};
+        if (kt < n_tiles) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kt * 16 + l16) * kQS + g * 16 + i * 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bq[i * 4 + j], acc, 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] = acc[r];
+      }
+    }
+    // ---- masked softmax over the keys of query q ------------------------------------------
+    const bool q_ok = q < seq_len;
+    const T* mrow = attr_mask + ((size_t)b * seq_len + (q_ok ? q : 0)) * seq_len;
+    float mx = 0.f;                          // clamp of the maximum at 0
+    const bool vec_mask = (seq_len & 3) == 0;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) {
+      const int key0 = kt * 16 + g * 4;
+      float mval[4] = {0.f, 0.f, 0.f, 0.f};
+      if (vec_mask) {
+        if (key0 < seq_len) {
+          typedef T mask4 __attribute__((ext_vector_type(4)));
+          const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + key0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) mval[r] = (float)m4[r];
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (key0 + r < seq_len) mval[r] = (float)mrow[key0 + r];
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        // keys beyond seq_len do not exist
+        const float tv = key0 + r < seq_len ? s[kt][r] * scaler + (1.0f - mval[r]) * -10000.0f : -INFINITY;
+        s[kt][r] = tv;
+        mx = fmaxf(mx, tv);
+      }
+    }
+    mx = xor_lanes_16_32_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[kt][r] = __builtin_amdgcn_exp2f((s[kt][r] - mx) * kLog2e);
+        sum += s[kt][r];
+      }
+    sum = xor_lanes_16_32_sum(sum) + 1e-6f;
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
+    // ---- O^T = V^T P^T --------------------------------------------------------------------
+    float4v o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int ks = 0; ks < NKT / 2; ++ks) {
+        if (2 * ks < n_tiles) {
+          half8 p;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            p[r] = f2h(s[2 * ks][r]);
+            p[4 + r] = f2h(s[2 * ks + 1][r]);
+          }
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) {
+            const T* vrow = Vt + (dt * 16 + l16) * kVS + ks * 32 + g * 4;
+            const half4 lo = *reinterpret_cast<const half4*>(vrow);
+            const half4 hi = *reinterpret_cast<const half4*>(vrow + 16);
+            half8 a;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              a[r] = lo[r];
+              a[4 + r] = hi[r];
+            }
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, p, o[dt], 0, 0, 0);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        if (kt < n_tiles) {
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) {
+            const float4v a4 = *reinterpret_cast<const float4v*>(Vt + (dt * 16 + l16) * kVS + kt * 16 + g * 4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[kt][r], o[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    // ---- write the lane's 4x4 features of its query's packed row --------------------------
+    const int tq = q < kSp ? tok_of_pos[q] : -1;
+    if (tq >= 0) {
+      T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        typedef T out4 __attribute__((ext_vector_type(4)));
+        out4 v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = (T)o[dt][r];
+        *reinterpret_cast<out4*>(orow + dt * 16) = v;
+      }
+    }
+  }
+}
+
+template <typename T, int NKT>
+void attention_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
+                      void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
+                      float scaler, hipStream_t stream) {
+  using Sm = AttnSmem<T, NKT>;
+  auto kern = attention_kernel<T, NKT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)Sm::kBytes);
+    attr_set = true;
+  }
+  dim3 grid(heads, batch);
+  kern<<<grid, kAttnThreads, Sm::kBytes, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
+                                                   (const T*)attr_mask, (T*)dst, seq_start, word_idx, seq_len, heads,
+                                                   scaler);
+}
+
+template <typename T>
+void attention_dispatch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
+                        void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
+                        float scaler, hipStream_t stream) {
+  if (seq_len <= 32)
+    attention_launch<T, 2>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                           scaler, stream);
+  else if (seq_len <= 64)
+    attention_launch<T, 4>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                           scaler, stream);
+  else
+    attention_launch<T, 8>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                           scaler, stream);
+}
+
+}  // namespace
+
+void launch_qkv_bias_pad(DType t, const void* Q, const void* bQ, const void* K, const void* bK, const void* V,
+                         const void* bV, void* q_buf, void* k_buf, void* v_buf, const int32_t* seq_start,
+                         const int32_t* word_idx, int batch, int seq_len, int heads, int d, hipStream_t stream) {
+  dim3 grid(batch, 3);
+  if (t == DType::F32)
+    qkv_bias_pad_kernel<float><<<grid, kPadThreads, 0, stream>>>(
+        (const float*)Q, (const float*)bQ, (const float*)K, (const float*)bK, (const float*)V, (const float*)bV,
+        (float*)q_buf, (float*)k_buf, (float*)v_buf, seq_start, word_idx, seq_len, heads, d);
+  else
+    qkv_bias_pad_kernel<_Float16><<<grid, kPadThreads, 0, stream>>>(
+        (const _Float16*)Q, (const _Float16*)bQ, (const _Float16*)K, (const _Float16*)bK, (const _Float16*)V,
+        (const _Float16*)bV, (_Float16*)q_buf, (_Float16*)k_buf, (_Float16*)v_buf, seq_start, word_idx, seq_len, heads,
+        d);
+}
+
+void launch_softmax(DType t, void* qk, const void* attr_mask, int batch, int heads, int seq_len, float scaler,
+                    hipStream_t stream) {
+  const int rows = batch * heads * seq_len;
+  const int grid = (rows + kSmThreads / kWave - 1) / (kSmThreads / kWave);
+  if (t == DType::F32)
+    softmax_kernel<float><<<grid, kSmThreads, 0, stream>>>((float*)qk, (const float*)attr_mask, rows, heads, seq_len,
+                                                           scaler);
+  else
+    softmax_kernel<_Float16><<<grid, kSmThreads, 0, stream>>>((_Float16*)qk, (const _Float16*)attr_mask, rows, heads,
+                                                              seq_len, scaler);
+}
+
+void launch_transpose_rm_padding(DType t, const void* src, void* dst, const int32_t* rows_dev, int rows_bound,
+                                 int batch, int seq_len, int heads, int d, const int32_t* batch_idx,
+                                 const int32_t* word_idx, hipStream_t stream) {
+  (void)batch;
+  const int cpd = (int)((size_t)d * elem_size(t) / 16);
+  const long total = (long)rows_bound * heads * cpd;
+  const int grid = (int)((total + 255) / 256);
+  if (grid == 0) return;
+  if (t == DType::F32)
+    transpose_rm_padding_kernel<float><<<grid, 256, 0, stream>>>((const float*)src, (float*)dst, rows_dev, rows_bound,
+                                                                 seq_len, heads, cpd, batch_idx, word_idx);
+  else
+    transpose_rm_padding_kernel<_Float16><<<grid, 256, 0, stream>>>((const _Float16*)src, (_Float16*)dst, rows_dev,
+                                                                    rows_bound, seq_len, heads, cpd, batch_idx,
+                                                                    word_idx);
+}
+
+bool attention_supported(DType t, int seq_len, int d) {
+  (void)t;
+  return d == kD && seq_len >= 1 && seq_len <= 128;
+}
+
+void launch_attention(DType t, const void* q, const void* k, const void* v, int layout, int packed_ld,
+                      const void* attr_mask, void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch,
+                      int seq_len, int heads, int d, float scaler, hipStream_t stream) {
+  (void)d;
+  if (t == DType::F32)
+    attention_dispatch<float>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                              scaler, stream);
+  else
+    attention_dispatch<_Float16>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len,
+                                 heads, scaler, stream);
+}
+
+}  // namespace et

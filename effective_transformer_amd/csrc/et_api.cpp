@@ -1,0 +1,466 @@
+// C ABI of libet_hip.so: argument validation, workspace carve-up and launch order of the three
+// ops (reference host side: tf_op/bert_transformer_op.cu.cc:33-373) plus the kernel-level entry
+// points.  No call allocates device memory; a handle serialises its calls with a mutex like the
+// reference's layer op does (tf_op/bert_transformer_op.cc:213).
+#include "../../include/et.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "kernels.hpp"
+
+struct et_context {
+  int device = 0;
+  std::mutex mu;
+  std::string last_error;
+};
+
+namespace {
+
+thread_local std::string tls_error;
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+et_status fail(et_handle h, et_status s, const std::string& msg) {
+  std::string full = std::string("[ET][ERROR] ") + et_status_string(s) + ": " + msg;
+  if (h)
+    h->last_error = full;
+  else
+    tls_error = full;
+  return s;
+}
+
+et_status check_hip(et_handle h, hipError_t e, const char* what, const char* file, int line) {
+  if (e == hipSuccess) return ET_OK;
+  return fail(h, ET_RUNTIME_ERROR,
+              std::string(what) + ": " + hipGetErrorString(e) + " " + file + ":" + std::to_string(line));
+}
+
+et_status check_launch(et_handle h, const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return ET_OK;
+  return fail(h, ET_LAUNCH_FAILURE, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define ET_HIP(h, call)                                                        \
+  do {                                                                         \
+    et_status _s = check_hip((h), (call), #call, __FILE__, __LINE__);          \
+    if (_s != ET_OK) return _s;                                                \
+  } while (0)
+
+#define ET_REQUIRE(h, cond, msg)                                               \
+  do {                                                                         \
+    if (!(cond)) return fail((h), ET_INVALID_ARGUMENT, (msg));                 \
+  } while (0)
+
+bool dtype_ok(et_dtype d) { return d == ET_FP32 || d == ET_FP16; }
+et::DType to_dt(et_dtype d) { return d == ET_FP32 ? et::DType::F32 : et::DType::F16; }
+
+struct LayerWs {
+  size_t qkv, ctx, attn, inter, seq, total;
+};
+
+LayerWs layer_ws(et_dtype dtype, int B, int S, int heads, int d) {
+  const size_t e = dtype == ET_FP32 ? 4 : 2;
+  const size_t rows = (size_t)B * S, H = (size_t)heads * d;
+  LayerWs w;
+  size_t off = 0;
+  w.qkv = off;   off += align_up(rows * 3 * H * e, 256);
+  w.ctx = off;   off += align_up(rows * H * e, 256);
+  w.attn = off;  off += align_up(rows * H * e, 256);
+  w.inter = off; off += align_up(rows * 4 * H * e, 256);
+  w.seq = off;   off += align_up(((size_t)B + 1) * sizeof(int32_t), 256);
+  w.total = off;
+  return w;
+}
+
+// Guard that makes the handle's device current and serialises calls on the handle.
+struct Scope {
+  std::lock_guard<std::mutex> lock;
+  explicit Scope(et_handle h) : lock(h->mu) {}
+};
+
+et_status enter(et_handle h) {
+  if (!h) return fail(nullptr, ET_INVALID_ARGUMENT, "null handle");
+  return check_hip(h, hipSetDevice(h->device), "hipSetDevice", __FILE__, __LINE__);
+}
+
+et_status dims_ok(et_handle h, int B, int S, int heads, int d) {
+  ET_REQUIRE(h, B >= 1 && S >= 1 && heads >= 1 && d >= 1, "batch_size, seq_len, head_num, size_per_head must be >= 1");
+  ET_REQUIRE(h, (long)B * S < (1L << 30), "batch_size * seq_len too large");
+  return ET_OK;
+}
+
+float softmax_scaler(et_dtype dtype, int d) {
+  float s = 1.0f / sqrtf((float)d);
+  if (dtype == ET_FP16) s = (float)(_Float16)s;   // the reference holds the scaler in the element type
+  return s;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* et_status_string(et_status s) {
+  switch (s) {
+    case ET_OK: return "ET_OK";
+    case ET_INVALID_ARGUMENT: return "ET_INVALID_ARGUMENT";
+    case ET_WORKSPACE_TOO_SMALL: return "ET_WORKSPACE_TOO_SMALL";
+    case ET_UNSUPPORTED: return "ET_UNSUPPORTED";
+    case ET_LAUNCH_FAILURE: return "ET_LAUNCH_FAILURE";
+    case ET_RUNTIME_ERROR: return "ET_RUNTIME_ERROR";
+  }
+  return "<unknown>";
+}
+
+int et_device_ok(int device) {
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) != hipSuccess) return 0;
+  return std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+}
+
+et_status et_create(et_handle* out, int device) {
+  if (!out) return fail(nullptr, ET_INVALID_ARGUMENT, "null output handle");
+  *out = nullptr;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess) return fail(nullptr, ET_RUNTIME_ERROR, std::string("hipGetDeviceCount: ") + hipGetErrorString(e));
+  if (device < 0 || device >= count) return fail(nullptr, ET_INVALID_ARGUMENT, "no such device");
+  if (!et_device_ok(device)) return fail(nullptr, ET_UNSUPPORTED, "device is not gfx950; the kernels are built for MI355X only");
+  et_context* c = new (std::nothrow) et_context();
+  if (!c) return fail(nullptr, ET_RUNTIME_ERROR, "out of host memory");
+  c->device = device;
+  *out = c;
+  return ET_OK;
+}
+
+et_status et_destroy(et_handle h) {
+  if (!h) return ET_OK;
+  delete h;
+  return ET_OK;
+}
+
+const char* et_last_error(et_handle h) { return h ? h->last_error.c_str() : tls_error.c_str(); }
+
+size_t et_input_workspace_bytes(int batch_size, int seq_len) {
+  if (batch_size < 1 || seq_len < 1) return 0;
+  return align_up((et::scan_scratch_words(batch_size * seq_len) + 1) * sizeof(int32_t), 256);
+}
+
+size_t et_layer_workspace_bytes(et_dtype dtype, int batch_size, int seq_len, int head_num, int size_per_head) {
+  if (batch_size < 1 || seq_len < 1 || head_num < 1 || size_per_head < 1 || !dtype_ok(dtype)) return 0;
+  return layer_ws(dtype, batch_size, seq_len, head_num, size_per_head).total;
+}
+
+size_t et_seq_workspace_bytes(int batch_size) {
+  if (batch_size < 1) return 0;
+  return align_up(((size_t)batch_size + 1) * sizeof(int32_t), 256);
+}
+
+et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask, void* to_tensor,
+                   int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx, int batch_size, int seq_len,
+                   int head_num, int size_per_head, void* workspace, size_t workspace_bytes, void* stream,
+                   int32_t* valid_word_num_host) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, from_tensor && mask && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  ET_REQUIRE(h, workspace != nullptr, "null workspace");
+  if (workspace_bytes < et_input_workspace_bytes(batch_size, seq_len))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "et_input needs et_input_workspace_bytes(batch_size, seq_len)");
+  const size_t row_bytes = (size_t)head_num * size_per_head * et::elem_size(to_dt(dtype));
+  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
+  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+    return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  et::launch_scan_index(mask, batch_size * seq_len, nullptr, batch_idx, word_idx, valid_word_num_dev, seq_len,
+                        (int32_t*)workspace, st);
+  if ((s = check_launch(h, "mask scan")) != ET_OK) return s;
+  et::launch_compress_rows(from_tensor, to_tensor, batch_idx, word_idx, valid_word_num_dev, nullptr, nullptr,
+                           batch_size, seq_len, (int)row_bytes, st);
+  if ((s = check_launch(h, "compress")) != ET_OK) return s;
+  if (valid_word_num_host) {
+    ET_HIP(h, hipMemcpyAsync(valid_word_num_host, valid_word_num_dev, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    ET_HIP(h, hipStreamSynchronize(st));
+  }
+  return ET_OK;
+}
+
+et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const void* from_tensor,
+                   const void* to_tensor, const void* attr_mask, const int32_t* valid_word_num_dev,
+                   const int32_t* batch_idx, const int32_t* word_idx, void* out, int batch_size, int from_seq_len,
+                   int to_seq_len, int head_num, int size_per_head, int valid_word_num_hint, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, from_seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, from_seq_len == to_seq_len, "only support from_seq_len == to_seq_len");
+  ET_REQUIRE(h, w != nullptr, "null weights");
+  ET_REQUIRE(h, w->attr_kernel_Q && w->attr_kernel_K && w->attr_kernel_V && w->attr_bias_Q && w->attr_bias_K &&
+                    w->attr_bias_V && w->attr_output_kernel && w->attr_output_bias && w->attr_output_layernorm_gamma &&
+                    w->attr_output_layernorm_beta && w->inter_kernel && w->inter_bias && w->output_kernel &&
+                    w->output_bias && w->output_layernorm_gamma && w->output_layernorm_beta,
+             "null weight pointer");
+  ET_REQUIRE(h, from_tensor && to_tensor && attr_mask && valid_word_num_dev && batch_idx && word_idx && out,
+             "null tensor pointer");
+  ET_REQUIRE(h, out != from_tensor && out != to_tensor, "out must not alias from_tensor / to_tensor");
+  ET_REQUIRE(h, workspace != nullptr, "null workspace");
+  const int B = batch_size, S = from_seq_len, H = head_num * size_per_head, F = 4 * H;
+  ET_REQUIRE(h, valid_word_num_hint >= -1 && valid_word_num_hint <= B * S, "valid_word_num_hint out of range");
+  const LayerWs ws = layer_ws(dtype, B, S, head_num, size_per_head);
+  if (workspace_bytes < ws.total) return fail(h, ET_WORKSPACE_TOO_SMALL, "et_layer needs et_layer_workspace_bytes(...)");
+  const et::DType dt = to_dt(dtype);
+  if (!et::attention_supported(dt, S, size_per_head))
+    return fail(h, ET_UNSUPPORTED, "attention kernel supports size_per_head == 64 and seq_len <= 128");
+  if (!et::gemm_supported(dt, H, H, 3) || !et::gemm_supported(dt, F, H, 1) || !et::gemm_supported(dt, H, F, 1))
+    return fail(h, ET_UNSUPPORTED, "hidden size not supported by the GEMM kernels");
+  if (!et::bias_gelu_supported(dt, F) || !et::bias_residual_layernorm_supported(dt, H))
+    return fail(h, ET_UNSUPPORTED, "hidden size not supported by the row kernels");
+  if (valid_word_num_hint == 0) return ET_OK;
+  const int rows = valid_word_num_hint > 0 ? valid_word_num_hint : B * S;
+  const int32_t* T = valid_word_num_dev;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t e = et::elem_size(dt);
+  char* base = (char*)workspace;
+  void* qkv = base + ws.qkv;
+  void* ctx = base + ws.ctx;
+  void* attn = base + ws.attn;
+  void* inter = base + ws.inter;
+  int32_t* seq_start = (int32_t*)(base + ws.seq);
+
+  et::launch_seq_start(batch_idx, T, rows, B, seq_start, st);
+  // Q = from.Wq + bq, K = to.Wk + bk, V = to.Wv + bv into one [T,3H] buffer (bert_transformer_op.cu.cc:105-156)
+  et::GemmGroups g3;
+  g3.groups = 3;
+  g3.A[0] = from_tensor; g3.A[1] = to_tensor; g3.A[2] = to_tensor;
+  g3.B[0] = w->attr_kernel_Q; g3.B[1] = w->attr_kernel_K; g3.B[2] = w->attr_kernel_V;
+  g3.bias[0] = w->attr_bias_Q; g3.bias[1] = w->attr_bias_K; g3.bias[2] = w->attr_bias_V;
+  et::launch_gemm(dt, g3, qkv, 3 * H, rows, H, H, T, st);
+  if ((s = check_launch(h, "QKV projection")) != ET_OK) return s;
+  // QK^T, softmax, PV, un-pad (:159-192)
+  et::launch_attention(dt, qkv, (char*)qkv + (size_t)H * e, (char*)qkv + (size_t)2 * H * e, 1, 3 * H, attr_mask, ctx,
+                       seq_start, word_idx, B, S, head_num, size_per_head, softmax_scaler(dtype, size_per_head), st);
+  if ((s = check_launch(h, "attention")) != ET_OK) return s;
+  // attention output projection + bias + residual(from_tensor) + LayerNorm (:195-213)
+  et::GemmGroups g1;
+  g1.groups = 1;
+  g1.A[0] = ctx; g1.B[0] = w->attr_output_kernel; g1.bias[0] = nullptr;
+  et::launch_gemm(dt, g1, attn, H, rows, H, H, T, st);
+  et::launch_bias_residual_layernorm(dt, attn, from_tensor, w->attr_output_bias, w->attr_output_layernorm_gamma,
+                                     w->attr_output_layernorm_beta, rows, H, T, st);
+  if ((s = check_launch(h, "attention output")) != ET_OK) return s;
+  // FFN up + bias + GELU (:215-227)
+  g1.A[0] = attn; g1.B[0] = w->inter_kernel;
+  et::launch_gemm(dt, g1, inter, F, rows, F, H, T, st);
+  et::launch_bias_gelu(dt, inter, w->inter_bias, rows, F, T, st);
+  if ((s = check_launch(h, "FFN up")) != ET_OK) return s;
+  // FFN down + bias + residual(LN1 output) + LayerNorm (:229-247)
+  g1.A[0] = inter; g1.B[0] = w->output_kernel;
+  et::launch_gemm(dt, g1, out, H, rows, H, F, T, st);
+  et::launch_bias_residual_layernorm(dt, out, attn, w->output_bias, w->output_layernorm_gamma,
+                                     w->output_layernorm_beta, rows, H, T, st);
+  if ((s = check_launch(h, "FFN down")) != ET_OK) return s;
+  return ET_OK;
+}
+
+et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* valid_word_num_dev,
+                    const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor, int batch_size, int seq_len,
+                    int head_num, int size_per_head, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  return et_restore(h, dtype, to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size, seq_len,
+                    head_num * size_per_head, stream);
+}
+
+et_status et_exclusive_scan(et_handle h, int32_t* d_out, const int32_t* d_in, int length, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, d_out && d_in, "null tensor pointer");
+  ET_REQUIRE(h, length >= 1 && length < (1 << 30), "length out of range");
+  ET_REQUIRE(h, workspace != nullptr, "null workspace");
+  if (workspace_bytes < et_input_workspace_bytes(1, length))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "et_exclusive_scan needs et_input_workspace_bytes(1, length)");
+  et::launch_scan_index(d_in, length, d_out, nullptr, nullptr, nullptr, 0, (int32_t*)workspace, (hipStream_t)stream);
+  return check_launch(h, "exclusive scan");
+}
+
+et_status et_compress(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask,
+                      const int32_t* prefix_sum, void* to_tensor, int32_t* batch_idx, int32_t* word_idx,
+                      int batch_size, int seq_len, int hidden_dim, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
+  ET_REQUIRE(h, from_tensor && mask && prefix_sum && to_tensor && batch_idx && word_idx, "null tensor pointer");
+  const size_t row_bytes = (size_t)hidden_dim * et::elem_size(to_dt(dtype));
+  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
+  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+    return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  et::launch_index_from_prefix(mask, prefix_sum, batch_idx, word_idx, batch_size, seq_len, st);
+  et::launch_compress_rows(from_tensor, to_tensor, batch_idx, word_idx, nullptr, prefix_sum, mask, batch_size, seq_len,
+                           (int)row_bytes, st);
+  return check_launch(h, "compress");
+}
+
+et_status et_restore(et_handle h, et_dtype dtype, void* to_tensor, const void* from_tensor, const int32_t* batch_idx,
+                     const int32_t* word_idx, const int32_t* valid_word_num_dev, int batch_size, int seq_len,
+                     int hidden_dim, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
+  ET_REQUIRE(h, from_tensor && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  const size_t row_bytes = (size_t)hidden_dim * et::elem_size(to_dt(dtype));
+  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
+  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+    return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
+  et::launch_restore_rows(to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size, seq_len,
+                          (int)row_bytes, (hipStream_t)stream);
+  return check_launch(h, "restore");
+}
+
+et_status et_add_bias_act(et_handle h, et_dtype dtype, void* out, const void* bias, int m, int n,
+                          const int32_t* m_dev, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  ET_REQUIRE(h, out && bias, "null tensor pointer");
+  ET_REQUIRE(h, m >= 0 && n >= 1, "bad dimensions");
+  if (!et::bias_gelu_supported(to_dt(dtype), n)) return fail(h, ET_UNSUPPORTED, "row bytes must be a multiple of 16");
+  if (m == 0) return ET_OK;
+  et::launch_bias_gelu(to_dt(dtype), out, bias, m, n, m_dev, (hipStream_t)stream);
+  return check_launch(h, "bias + gelu");
+}
+
+et_status et_add_bias_input_layernorm(et_handle h, et_dtype dtype, void* out, const void* input, const void* bias,
+                                      const void* gamma, const void* beta, int m, int n, const int32_t* m_dev,
+                                      void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  ET_REQUIRE(h, out && input && bias && gamma && beta, "null tensor pointer");
+  ET_REQUIRE(h, m >= 0 && n >= 1, "bad dimensions");
+  if (!et::bias_residual_layernorm_supported(to_dt(dtype), n))
+    return fail(h, ET_UNSUPPORTED, "row length not supported by the LayerNorm kernel");
+  if (m == 0) return ET_OK;
+  et::launch_bias_residual_layernorm(to_dt(dtype), out, input, bias, gamma, beta, m, n, m_dev, (hipStream_t)stream);
+  return check_launch(h, "bias + residual + layernorm");
+}
+
+et_status et_add_qkv_bias_padding(et_handle h, et_dtype dtype, const void* Q, const void* bias_Q, const void* K,
+                                  const void* bias_K, const void* V, const void* bias_V, void* q_buf, void* k_buf,
+                                  void* v_buf, const int32_t* valid_word_num_dev, int batch_size, int seq_len,
+                                  int head_num, int size_per_head, const int32_t* batch_idx, const int32_t* word_idx,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, Q && K && V && bias_Q && bias_K && bias_V && q_buf && k_buf && v_buf && valid_word_num_dev &&
+                    batch_idx && word_idx,
+             "null tensor pointer");
+  ET_REQUIRE(h, workspace != nullptr, "null workspace");
+  if (workspace_bytes < et_seq_workspace_bytes(batch_size))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
+  if (((size_t)size_per_head * et::elem_size(to_dt(dtype))) % 16 != 0 || seq_len > 1024)
+    return fail(h, ET_UNSUPPORTED, "size_per_head bytes must be a multiple of 16 and seq_len <= 1024");
+  hipStream_t st = (hipStream_t)stream;
+  et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, (int32_t*)workspace, st);
+  et::launch_qkv_bias_pad(to_dt(dtype), Q, bias_Q, K, bias_K, V, bias_V, q_buf, k_buf, v_buf, (int32_t*)workspace,
+                          word_idx, batch_size, seq_len, head_num, size_per_head, st);
+  return check_launch(h, "qkv bias + padding");
+}
+
+et_status et_softmax(et_handle h, et_dtype dtype, void* qk_buf, const void* attr_mask, int batch_size, int head_num,
+                     int seq_len, float scaler, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, 1)) != ET_OK) return s;
+  ET_REQUIRE(h, qk_buf && attr_mask, "null tensor pointer");
+  if (seq_len > 512) return fail(h, ET_UNSUPPORTED, "softmax kernel supports seq_len <= 512");
+  et::launch_softmax(to_dt(dtype), qk_buf, attr_mask, batch_size, head_num, seq_len, scaler, (hipStream_t)stream);
+  return check_launch(h, "softmax");
+}
+
+et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, void* dst,
+                                  const int32_t* valid_word_num_dev, int batch_size, int seq_len, int head_num,
+                                  int size_per_head, const int32_t* batch_idx, const int32_t* word_idx, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, src && dst && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  if (((size_t)size_per_head * et::elem_size(to_dt(dtype))) % 16 != 0)
+    return fail(h, ET_UNSUPPORTED, "size_per_head bytes must be a multiple of 16");
+  et::launch_transpose_rm_padding(to_dt(dtype), src, dst, valid_word_num_dev, batch_size * seq_len, batch_size,
+                                  seq_len, head_num, size_per_head, batch_idx, word_idx, (hipStream_t)stream);
+  return check_launch(h, "transpose + remove padding");
+}
+
+et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v, int qkv_layout,
+                       int packed_ld, const void* attr_mask, void* dst, const int32_t* valid_word_num_dev,
+                       int batch_size, int seq_len, int head_num, int size_per_head, const int32_t* batch_idx,
+                       const int32_t* word_idx, void* workspace, size_t workspace_bytes, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, q && k && v && attr_mask && dst && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  ET_REQUIRE(h, qkv_layout == 0 || qkv_layout == 1, "qkv_layout must be 0 (padded) or 1 (packed)");
+  ET_REQUIRE(h, qkv_layout == 0 || packed_ld >= head_num * size_per_head, "packed_ld smaller than the hidden size");
+  ET_REQUIRE(h, workspace != nullptr, "null workspace");
+  if (workspace_bytes < et_seq_workspace_bytes(batch_size))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
+  if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
+    return fail(h, ET_UNSUPPORTED, "attention kernel supports size_per_head == 64 and seq_len <= 128");
+  if (qkv_layout == 1 && ((size_t)packed_ld * et::elem_size(to_dt(dtype))) % 16 != 0)
+    return fail(h, ET_UNSUPPORTED, "packed_ld bytes must be a multiple of 16");
+  hipStream_t st = (hipStream_t)stream;
+  et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, (int32_t*)workspace, st);
+  et::launch_attention(to_dt(dtype), q, k, v, qkv_layout, packed_ld, attr_mask, dst, (int32_t*)workspace, word_idx,
+                       batch_size, seq_len, head_num, size_per_head, softmax_scaler(dtype, size_per_head), st);
+  return check_launch(h, "attention");
+}
+
+et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias, int m, int n,
+                  int k, const int32_t* m_dev, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  ET_REQUIRE(h, A && B && C, "null tensor pointer");
+  ET_REQUIRE(h, m >= 0 && n >= 1 && k >= 1, "bad dimensions");
+  if (!et::gemm_supported(to_dt(dtype), n, k, 1))
+    return fail(h, ET_UNSUPPORTED, dtype == ET_FP16 ? "fp16 GEMM needs k % 64 == 0 and n % 8 == 0"
+                                                     : "fp32 GEMM needs k % 16 == 0 and n % 4 == 0");
+  if (m == 0) return ET_OK;
+  et::GemmGroups g;
+  g.groups = 1;
+  g.A[0] = A; g.B[0] = B; g.bias[0] = bias;
+  et::launch_gemm(to_dt(dtype), g, C, n, m, n, k, m_dev, (hipStream_t)stream);
+  return check_launch(h, "gemm");
+}
+
+}  // extern "C"

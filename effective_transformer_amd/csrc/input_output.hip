@@ -1,0 +1,278 @@
+// Input / output side of the padding-free encoder on gfx950:
+//   mask prefix sum + packed-token index build   (reference: cuda/cuda_kernels.cu:472-718,
+//                                                 tf_op/bert_transformer_op.cu.cc:266-331)
+//   compress [B,S,H] -> [T,H]                    (cuda/cuda_kernels.cu:278-384)
+//   restore  [T,H]  -> [B,S,H] with zero fill    (cuda/cuda_kernels.cu:389-468,
+//                                                 tf_op/bert_transformer_op.cu.cc:351-360)
+// All of it is HBM-bound byte and integer work: the scan runs on 64-lane DPP prefix sums, the
+// row movers use one 128-bit access per lane on a flattened (row, 16-byte chunk) index space so
+// that every lane of every wavefront carries data.
+#include "et_device.hpp"
+#include "kernels.hpp"
+
+namespace et {
+
+namespace {
+
+constexpr int kScanThreads = 256;
+constexpr int kScanWaves = kScanThreads / kWave;
+
+inline int scan_tile_for(int length) {
+  // at most 1024 tiles, so that one workgroup can reduce the tile totals in front of it
+  int tile = 1024;
+  long need = ((long)length + 1023) / 1024;
+  if (need > tile) tile = (int)((need + kScanThreads - 1) / kScanThreads) * kScanThreads;
+  return tile;
+}
+
+__device__ __forceinline__ int block_sum_i32(int v, int* lds /* >= kScanWaves ints */) {
+  int w = wave_sum_i32(v);
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();                       // protect lds from a previous use
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = w;
+  __syncthreads();
+  int total = 0;
+#pragma unroll
+  for (int i = 0; i < kScanWaves; ++i) total += lds[i];
+  return total;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(const int32_t* __restrict__ in, int n, int tile,
+                                                                       int32_t* __restrict__ sums) {
+  __shared__ int lds[kScanWaves];
+  const int begin = blockIdx.x * tile;
+  const int end = min(n, begin + tile);
+  int acc = 0;
+  for (int i = begin + threadIdx.x; i < end; i += kScanThreads) acc += in[i];
+  int total = block_sum_i32(acc, lds);
+  if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+// One workgroup per tile: adds up the totals of the tiles in front of it, then walks its tile
+// in steps of 256 elements with a DPP scan per wavefront.
+__global__ __launch_bounds__(kScanThreads) void scan_index_kernel(const int32_t* __restrict__ in, int n, int tile,
+                                                                   const int32_t* __restrict__ sums,
+                                                                   int32_t* __restrict__ prefix_out,
+                                                                   int32_t* __restrict__ batch_idx,
+                                                                   int32_t* __restrict__ word_idx,
+                                                                   int32_t* __restrict__ valid_word_num, int seq_len) {
+  __shared__ int lds[kScanWaves];
+  __shared__ int wave_tot[kScanWaves];
+  int part = 0;
+  for (int i = threadIdx.x; i < (int)blockIdx.x; i += kScanThreads) part += sums[i];
+  int carry = block_sum_i32(part, lds);
+
+  const int begin = blockIdx.x * tile;
+  const int end = min(n, begin + tile);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  for (int c0 = begin; c0 < end; c0 += kScanThreads) {
+    const int idx = c0 + threadIdx.x;
+    const int v = idx < end ? in[idx] : 0;
+    const int inc = wave_inclusive_scan_i32(v);
+    if (lane == kWave - 1) wave_tot[wave] = inc;
+    __syncthreads();
+    int before = 0, chunk = 0;
+#pragma unroll
+    for (int w = 0; w < kScanWaves; ++w) {
+      const int t = wave_tot[w];
+      before += (w < wave) ? t : 0;
+      chunk += t;
+    }
+    const int excl = carry + before + inc - v;
+    if (idx < end) {
+      if (prefix_out) prefix_out[idx] = excl;
+      if (seq_len > 0) {
+        if (v > 0) {                       // the reference tests mask > 0.5 (cuda_kernels.cu:292)
+          const int b = idx / seq_len;
+          batch_idx[excl] = b;
+          word_idx[excl] = idx - b * seq_len;
+        }
+        // T = prefix[last] + (mask[last] == 1)   (bert_transformer_op.cu.cc:306-315)
+        if (idx == n - 1) *valid_word_num = excl + (v == 1 ? 1 : 0);
+      }
+    }
+    carry += chunk;
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(256) void index_from_prefix_kernel(const int32_t* __restrict__ mask,
+                                                                const int32_t* __restrict__ prefix,
+                                                                int32_t* __restrict__ batch_idx,
+                                                                int32_t* __restrict__ word_idx, int n, int seq_len) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  if (mask[idx] > 0) {
+    const int t = prefix[idx];
+    const int b = idx / seq_len;
+    batch_idx[t] = b;
+    word_idx[t] = idx - b * seq_len;
+  }
+}
+
+constexpr int kMoveThreads = 256;
+constexpr int kMoveUnroll = 4;
+
+// Gather of packed rows: flattened over (packed row, 16-byte chunk).
+__global__ __launch_bounds__(kMoveThreads) void compress_rows_kernel(
+    const u32x4* __restrict__ from, u32x4* __restrict__ to, const int32_t* __restrict__ batch_idx,
+    const int32_t* __restrict__ word_idx, const int32_t* __restrict__ rows_dev, const int32_t* __restrict__ prefix,
+    const int32_t* __restrict__ mask, int n_pos, int seq_len, fastdiv cpr) {
+  int T;
+  if (rows_dev) {
+    T = *rows_dev;
+  } else {
+    T = prefix[n_pos - 1] + (mask[n_pos - 1] == 1 ? 1 : 0);
+  }
+  T = min(T, n_pos);
+  const uint32_t total = (uint32_t)T * cpr.d;
+  const uint32_t base = blockIdx.x * (kMoveThreads * kMoveUnroll) + threadIdx.x;
+  u32x4 val[kMoveUnroll];
+  uint32_t dst[kMoveUnroll];
+#pragma unroll
+  for (int u = 0; u < kMoveUnroll; ++u) {
+    const uint32_t i = base + u * kMoveThreads;
+    dst[u] = i;
+    if (i < total) {
+      const uint32_t t = div_by(i, cpr);
+      const uint32_t c = i - t * cpr.d;
+      const uint32_t src_row = (uint32_t)batch_idx[t] * (uint32_t)seq_len + (uint32_t)word_idx[t];
+      val[u] = from[(size_t)src_row * cpr.d + c];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kMoveUnroll; ++u)
+    if (dst[u] < total) to[dst[u]] = val[u];
+}
+
+constexpr int kRestorePos = 32;   // padded positions per workgroup
+
+// One pass over the padded output: every 16-byte chunk of [B*S, row] is written exactly once,
+// either from its packed row or with zeros.  The packed row of a padded position is found
+// without scratch memory: keys b*S+s are ascending in t, so a 64-way search by one wavefront
+// locates the first packed row at or after the workgroup's first position and the next
+// kRestorePos keys cover everything that can land in the workgroup's window.
+__global__ __launch_bounds__(kMoveThreads) void restore_rows_kernel(
+    u32x4* __restrict__ to, const u32x4* __restrict__ from, const int32_t* __restrict__ batch_idx,
+    const int32_t* __restrict__ word_idx, const int32_t* __restrict__ rows_dev, int n_pos, int seq_len, int cpr) {
+  __shared__ int inv[kRestorePos];
+  __shared__ int t0_sh;
+  const int p0 = blockIdx.x * kRestorePos;
+  const int T = min(*rows_dev, n_pos);
+  if (threadIdx.x < kRestorePos) inv[threadIdx.x] = -1;
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    int lo = 0, hi = T;                 // first t with key(t) >= p0 lies in [lo, hi]
+    while (hi > lo) {
+      const int len = hi - lo;
+      const int step = (len + kWave - 1) / kWave;
+      const int probe = lo + lane * step;
+      bool below = false;
+      if (probe < hi) below = (batch_idx[probe] * seq_len + word_idx[probe]) < p0;
+      const int c = __popcll(__ballot(below));
+      if (c == 0) {
+        hi = lo;
+      } else {
+        const int nlo = lo + (c - 1) * step + 1;
+        const int nhi = min(lo + c * step, hi);
+        lo = nlo;
+        hi = nhi;
+      }
+    }
+    if (lane == 0) t0_sh = lo;
+  }
+  __syncthreads();
+  const int t0 = t0_sh;
+  if (threadIdx.x < kRestorePos) {
+    const int t = t0 + threadIdx.x;
+    if (t < T) {
+      const int key = batch_idx[t] * seq_len + word_idx[t];
+      if (key >= p0 && key < p0 + kRestorePos) inv[key - p0] = t;
+    }
+  }
+  __syncthreads();
+  const int npos = min(kRestorePos, n_pos - p0);
+  const int total = npos * cpr;
+  for (int i0 = 0; i0 < total; i0 += kMoveThreads * kMoveUnroll) {
+    u32x4 val[kMoveUnroll];
+#pragma unroll
+    for (int u = 0; u < kMoveUnroll; ++u) {
+      const int i = i0 + u * kMoveThreads + threadIdx.x;
+      val[u] = u32x4{0u, 0u, 0u, 0u};
+      if (i < total) {
+        const int r = i / cpr;
+        const int c = i - r * cpr;
+        const int t = inv[r];
+        if (t >= 0) val[u] = from[(size_t)t * cpr + c];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kMoveUnroll; ++u) {
+      const int i = i0 + u * kMoveThreads + threadIdx.x;
+      if (i < total) to[(size_t)p0 * cpr + i] = val[u];
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restrict__ batch_idx,
+                                                        const int32_t* __restrict__ rows_dev, int rows_bound,
+                                                        int batch, int32_t* __restrict__ seq_start) {
+  const int T = rows_dev ? min(*rows_dev, rows_bound) : rows_bound;
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t > T) return;
+  const int prev = t == 0 ? -1 : batch_idx[t - 1];
+  const int cur = t == T ? batch : min(batch_idx[t], batch - 1);
+  const int last = t == T ? batch : cur;         // entries (prev, last] start at t
+  for (int b = prev + 1; b <= last; ++b) seq_start[b] = t;
+}
+
+}  // namespace
+
+size_t scan_scratch_words(int length) {
+  const int tile = scan_tile_for(length);
+  return (size_t)((length + tile - 1) / tile);
+}
+
+void launch_scan_index(const int32_t* in, int length, int32_t* prefix_out, int32_t* batch_idx, int32_t* word_idx,
+                       int32_t* valid_word_num, int seq_len, int32_t* scratch, hipStream_t stream) {
+  const int tile = scan_tile_for(length);
+  const int tiles = (length + tile - 1) / tile;
+  if (tiles > 1) scan_tile_sums_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, scratch);
+  scan_index_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, scratch, prefix_out, batch_idx, word_idx,
+                                                         valid_word_num, seq_len);
+}
+
+void launch_index_from_prefix(const int32_t* mask, const int32_t* prefix, int32_t* batch_idx, int32_t* word_idx,
+                              int batch, int seq_len, hipStream_t stream) {
+  const int n = batch * seq_len;
+  index_from_prefix_kernel<<<(n + 255) / 256, 256, 0, stream>>>(mask, prefix, batch_idx, word_idx, n, seq_len);
+}
+
+void launch_compress_rows(const void* from, void* to, const int32_t* batch_idx, const int32_t* word_idx,
+                          const int32_t* rows_dev, const int32_t* prefix, const int32_t* mask, int batch, int seq_len,
+                          int row_bytes, hipStream_t stream) {
+  const int n_pos = batch * seq_len;
+  const uint32_t cpr = (uint32_t)row_bytes / 16u;
+  const uint64_t chunks = (uint64_t)n_pos * cpr;
+  const uint32_t per_wg = kMoveThreads * kMoveUnroll;
+  const uint32_t grid = (uint32_t)((chunks + per_wg - 1) / per_wg);
+  compress_rows_kernel<<<grid, kMoveThreads, 0, stream>>>((const u32x4*)from, (u32x4*)to, batch_idx, word_idx,
+                                                          rows_dev, prefix, mask, n_pos, seq_len, make_fastdiv(cpr));
+}
+
+void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
+                         const int32_t* rows_dev, int batch, int seq_len, int row_bytes, hipStream_t stream) {
+  const int n_pos = batch * seq_len;
+  const int grid = (n_pos + kRestorePos - 1) / kRestorePos;
+  restore_rows_kernel<<<grid, kMoveThreads, 0, stream>>>((u32x4*)to, (const u32x4*)from, batch_idx, word_idx, rows_dev,
+                                                         n_pos, seq_len, row_bytes / 16);
+}
+
+void launch_seq_start(const int32_t* batch_idx, const int32_t* rows_dev, int rows_bound, int batch,
+                      int32_t* seq_start, hipStream_t stream) {
+  const int n = rows_bound + 1;
+  seq_start_kernel<<<(n + 255) / 256, 256, 0, stream>>>(batch_idx, rows_dev, rows_bound, batch, seq_start);
+}
+
+}  // namespace et

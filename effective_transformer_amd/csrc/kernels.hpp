@@ -1,0 +1,77 @@
+// Internal launcher interface between the C ABI (et_api.cpp) and the gfx950 kernels.
+// Every launcher enqueues on `stream` and returns; none allocates.  Row counts that live on
+// the device are passed as `rows_dev` (may be null) next to a host-side upper bound.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace et {
+
+enum class DType : int { F32 = 0, F16 = 1 };
+inline size_t elem_size(DType t) { return t == DType::F32 ? 4 : 2; }
+
+// ---- input_output.hip --------------------------------------------------------------------
+// Number of int32 words of scratch the scan needs for `length` elements.
+size_t scan_scratch_words(int length);
+// Exclusive prefix sum of `in`; optionally (seq_len > 0) also writes batch_idx / word_idx for
+// every element > 0 and the valid-token count.  prefix_out may be null.
+void launch_scan_index(const int32_t* in, int length, int32_t* prefix_out, int32_t* batch_idx,
+                       int32_t* word_idx, int32_t* valid_word_num, int seq_len, int32_t* scratch,
+                       hipStream_t stream);
+// batch_idx / word_idx from mask + an existing prefix sum.
+void launch_index_from_prefix(const int32_t* mask, const int32_t* prefix, int32_t* batch_idx,
+                              int32_t* word_idx, int batch, int seq_len, hipStream_t stream);
+// to[t,:] = from[batch_idx[t]*S + word_idx[t], :] for t < T.  T comes from *rows_dev when given,
+// otherwise from prefix[last] + (mask[last] == 1).
+void launch_compress_rows(const void* from, void* to, const int32_t* batch_idx, const int32_t* word_idx,
+                          const int32_t* rows_dev, const int32_t* prefix, const int32_t* mask,
+                          int batch, int seq_len, int row_bytes, hipStream_t stream);
+// to[B*S rows] = 0 at padding, from[t] at batch_idx[t]*S + word_idx[t]; indices ascending.
+void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
+                         const int32_t* rows_dev, int batch, int seq_len, int row_bytes, hipStream_t stream);
+// seq_start[b] = first packed row of sequence b, b in [0,B]; seq_start[B] = T.
+void launch_seq_start(const int32_t* batch_idx, const int32_t* rows_dev, int rows_bound, int batch,
+                      int32_t* seq_start, hipStream_t stream);
+
+// ---- row_kernels.hip ---------------------------------------------------------------------
+bool bias_gelu_supported(DType t, int n);
+void launch_bias_gelu(DType t, void* out, const void* bias, int m, int n, const int32_t* rows_dev,
+                      hipStream_t stream);
+bool bias_residual_layernorm_supported(DType t, int n);
+void launch_bias_residual_layernorm(DType t, void* out, const void* input, const void* bias,
+                                    const void* gamma, const void* beta, int m, int n,
+                                    const int32_t* rows_dev, hipStream_t stream);
+
+// ---- attention.hip -----------------------------------------------------------------------
+void launch_qkv_bias_pad(DType t, const void* Q, const void* bQ, const void* K, const void* bK,
+                         const void* V, const void* bV, void* q_buf, void* k_buf, void* v_buf,
+                         const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len,
+                         int heads, int d, hipStream_t stream);
+void launch_softmax(DType t, void* qk, const void* attr_mask, int batch, int heads, int seq_len,
+                    float scaler, hipStream_t stream);
+void launch_transpose_rm_padding(DType t, const void* src, void* dst, const int32_t* rows_dev,
+                                 int rows_bound, int batch, int seq_len, int heads, int d,
+                                 const int32_t* batch_idx, const int32_t* word_idx, hipStream_t stream);
+bool attention_supported(DType t, int seq_len, int d);
+// layout 0: padded [B,heads,S,d]; layout 1: packed rows with leading dimension packed_ld.
+void launch_attention(DType t, const void* q, const void* k, const void* v, int layout, int packed_ld,
+                      const void* attr_mask, void* dst, const int32_t* seq_start, const int32_t* word_idx,
+                      int batch, int seq_len, int heads, int d, float scaler, hipStream_t stream);
+
+// ---- gemm.hip ----------------------------------------------------------------------------
+// Up to three independent column groups share one launch (the Q/K/V projections): group g
+// computes C[:, g*n : (g+1)*n] = A[g] . B[g] (+ bias[g]) into a row-major C with leading
+// dimension ldc.  groups == 1 is the plain GEMM.
+struct GemmGroups {
+  const void* A[3];
+  const void* B[3];
+  const void* bias[3];
+  int groups;
+};
+bool gemm_supported(DType t, int n, int k, int groups);
+void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k,
+                 const int32_t* rows_dev, hipStream_t stream);
+
+}  // namespace et

@@ -1,0 +1,252 @@
+// Row kernels of the encoder layer on gfx950, both HBM-bound:
+//   out = gelu_tanh(out + bias)                       (reference: cuda/cuda_kernels.cu:29-51, 88-150)
+//   out = LayerNorm(out + input + bias) * gamma + beta (reference: cuda/cuda_kernels.cu:157-271)
+// Arithmetic and rounding points follow the reference: fp32 rows are computed in float; fp16
+// rows add in half (packed v_pk_add_f16), take statistics / the tanh polynomial in float and
+// round once on the way out.
+#include "et_device.hpp"
+#include "kernels.hpp"
+
+namespace et {
+
+namespace {
+
+// ------------------------------------------------------------------------------------------
+// bias + GELU.  0.5*(1+tanh(u)) is evaluated as 1/(1+exp(-2u)), which is the same function
+// without the cancellation of 1+tanh for negative u.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_cdf(float x, float x3) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x3);
+  // exp(-2u) = 2^(-2u*log2(e))
+  const float e = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);
+  return __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+constexpr int kGeluThreads = 128;
+constexpr int kGeluRows = 16;     // rows per workgroup
+constexpr int kGeluInFlight = 4;  // rows loaded before any is computed
+
+template <typename T> struct GeluChunk;
+
+template <> struct GeluChunk<float> {
+  float4v v;
+  __device__ __forceinline__ void apply(const GeluChunk<float>& b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float x = v[i] + b.v[i];
+      v[i] = x * gelu_cdf(x, x * x * x);
+    }
+  }
+};
+
+template <> struct GeluChunk<_Float16> {
+  half8 v;
+  __device__ __forceinline__ void apply(const GeluChunk<_Float16>& b) {
+    const half8 x = v + b.v;                 // __hadd2
+    const half8 x3 = x * (x * x);            // two half roundings (__hmul2 twice)
+    half8 cdf;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cdf[i] = f2h(gelu_cdf(h2f(x[i]), h2f(x3[i])));
+    v = x * cdf;
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(kGeluThreads) void bias_gelu_kernel(T* __restrict__ out, const T* __restrict__ bias, int m,
+                                                                 int cpr, const int32_t* __restrict__ rows_dev) {
+  using Chunk = GeluChunk<T>;
+  static_assert(sizeof(Chunk) == 16, "one 128-bit access per lane");
+  const int rows = rows_dev ? min(*rows_dev, m) : m;
+  const int c = blockIdx.x * kGeluThreads + threadIdx.x;
+  const int r0 = blockIdx.y * kGeluRows;
+  if (c >= cpr || r0 >= rows) return;
+  Chunk* base = reinterpret_cast<Chunk*>(out) + c;
+  const Chunk b = reinterpret_cast<const Chunk*>(bias)[c];
+  const int r1 = min(r0 + kGeluRows, rows);
+  for (int r = r0; r < r1; r += kGeluInFlight) {
+    Chunk x[kGeluInFlight];
+#pragma unroll
+    for (int u = 0; u < kGeluInFlight; ++u)
+      if (r + u < r1) x[u] = base[(size_t)(r + u) * cpr];
+#pragma unroll
+    for (int u = 0; u < kGeluInFlight; ++u)
+      if (r + u < r1) {
+        x[u].apply(b);
+        base[(size_t)(r + u) * cpr] = x[u];
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// bias + residual + LayerNorm: one wavefront per row, the row lives in registers between the
+// two statistics passes, both reductions are 64-lane DPP sums (no LDS, no barrier).
+// ------------------------------------------------------------------------------------------
+constexpr int kLnThreads = 256;
+constexpr int kLnWaves = kLnThreads / kWave;
+
+template <typename T, int VEC> struct RowVec;
+template <int VEC> struct RowVec<float, VEC> {
+  typedef float type __attribute__((ext_vector_type(VEC)));
+};
+template <int VEC> struct RowVec<_Float16, VEC> {
+  typedef _Float16 type __attribute__((ext_vector_type(VEC)));
+};
+
+// VEC elements per lane per access, ITERS accesses per row: the row has n <= 64*VEC*ITERS
+// elements, n % VEC == 0.
+template <typename T, int VEC, int ITERS>
+__global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
+    T* __restrict__ out, const T* __restrict__ input, const T* __restrict__ bias, const T* __restrict__ gamma,
+    const T* __restrict__ beta, int m, int n, const int32_t* __restrict__ rows_dev) {
+  using V = typename RowVec<T, VEC>::type;
+  const int rows = rows_dev ? min(*rows_dev, m) : m;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = blockIdx.x * kLnWaves + threadIdx.x / kWave;
+  const int nwaves = gridDim.x * kLnWaves;
+  const int vpr = n / VEC;                       // vectors per row
+
+  V b[ITERS], g[ITERS], be[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = lane + i * kWave;
+    if (c < vpr) {
+      b[i] = reinterpret_cast<const V*>(bias)[c];
+      g[i] = reinterpret_cast<const V*>(gamma)[c];
+      be[i] = reinterpret_cast<const V*>(beta)[c];
+    }
+  }
+  const float inv_n = 1.0f / (float)n;
+
+  for (int r = wave; r < rows; r += nwaves) {
+    V* orow = reinterpret_cast<V*>(out + (size_t)r * n);
+    const V* irow = reinterpret_cast<const V*>(input + (size_t)r * n);
+    V xo[ITERS], xi[ITERS];
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+      if (c < vpr) {
+        xo[i] = orow[c];
+        xi[i] = irow[c];
+      }
+    }
+    float x[ITERS][VEC];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+      // (out + input) + bias in the element type: float adds for fp32, two half roundings for fp16
+      const V s = (xo[i] + xi[i]) + b[i];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        x[i][j] = c < vpr ? (float)s[j] : 0.f;
+        sum += x[i][j];
+      }
+    }
+    const float mean = wave_sum(sum) * inv_n;
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float dlt = x[i][j] - mean;
+        sq += c < vpr ? dlt * dlt : 0.f;
+      }
+    }
+    const float rstd = __builtin_amdgcn_rsqf(wave_sum(sq) * inv_n + 1e-6f);
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+      if (c < vpr) {
+        V y;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) y[j] = (T)(((x[i][j] - mean) * rstd) * (float)g[i][j] + (float)be[i][j]);
+        orow[c] = y;
+      }
+    }
+  }
+}
+
+template <typename T>
+bool ln_pick(int n, int& vec, int& iters) {
+  const int max_vec = 16 / (int)sizeof(T);
+  for (int v = max_vec; v >= max_vec / 4 && v >= 1; v /= 2) {
+    if (n % v) continue;
+    const int it = (n / v + kWave - 1) / kWave;
+    if (it <= 8) {
+      vec = v;
+      iters = it;
+      return true;
+    }
+  }
+  return false;
+}
+
+template <typename T, int VEC>
+void ln_launch_iters(int iters, int grid, hipStream_t stream, T* out, const T* input, const T* bias, const T* gamma,
+                     const T* beta, int m, int n, const int32_t* rows_dev) {
+#define ET_LN_CASE(I)                                                                                          \
+  case I:                                                                                                      \
+    bias_residual_layernorm_kernel<T, VEC, I><<<grid, kLnThreads, 0, stream>>>(out, input, bias, gamma, beta, m, n, \
+                                                                               rows_dev);                      \
+    break;
+  switch (iters) {
+    ET_LN_CASE(1)
+    ET_LN_CASE(2)
+    ET_LN_CASE(3)
+    ET_LN_CASE(4)
+    ET_LN_CASE(5)
+    ET_LN_CASE(6)
+    ET_LN_CASE(7)
+    ET_LN_CASE(8)
+  }
+#undef ET_LN_CASE
+}
+
+template <typename T>
+void ln_launch(void* out, const void* input, const void* bias, const void* gamma, const void* beta, int m, int n,
+               const int32_t* rows_dev, hipStream_t stream) {
+  int vec = 0, iters = 0;
+  if (!ln_pick<T>(n, vec, iters)) return;
+  // enough wavefronts to fill 256 CUs several times over; rows beyond that are looped
+  const int grid = (int)min((long)(m + kLnWaves - 1) / kLnWaves, 256L * 8);
+  T* o = (T*)out;
+  const T *i = (const T*)input, *b = (const T*)bias, *g = (const T*)gamma, *be = (const T*)beta;
+  constexpr int MV = 16 / (int)sizeof(T);
+  if (vec == MV)
+    ln_launch_iters<T, MV>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
+  else if (vec == MV / 2)
+    ln_launch_iters<T, MV / 2>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
+  else
+    ln_launch_iters<T, MV / 4>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
+}
+
+}  // namespace
+
+bool bias_gelu_supported(DType t, int n) { return n > 0 && ((size_t)n * elem_size(t)) % 16 == 0; }
+
+void launch_bias_gelu(DType t, void* out, const void* bias, int m, int n, const int32_t* rows_dev, hipStream_t stream) {
+  const int cpr = (int)((size_t)n * elem_size(t) / 16);
+  dim3 grid((cpr + kGeluThreads - 1) / kGeluThreads, (m + kGeluRows - 1) / kGeluRows);
+  if (t == DType::F32)
+    bias_gelu_kernel<float><<<grid, kGeluThreads, 0, stream>>>((float*)out, (const float*)bias, m, cpr, rows_dev);
+  else
+    bias_gelu_kernel<_Float16><<<grid, kGeluThreads, 0, stream>>>((_Float16*)out, (const _Float16*)bias, m, cpr,
+                                                                  rows_dev);
+}
+
+bool bias_residual_layernorm_supported(DType t, int n) {
+  int vec, iters;
+  if (n <= 0) return false;
+  return t == DType::F32 ? ln_pick<float>(n, vec, iters) : ln_pick<_Float16>(n, vec, iters);
+}
+
+void launch_bias_residual_layernorm(DType t, void* out, const void* input, const void* bias, const void* gamma,
+                                    const void* beta, int m, int n, const int32_t* rows_dev, hipStream_t stream) {
+  if (t == DType::F32)
+    ln_launch<float>(out, input, bias, gamma, beta, m, n, rows_dev, stream);
+  else
+    ln_launch<_Float16>(out, input, bias, gamma, beta, m, n, rows_dev, stream);
+}
+
+}  // namespace et

@@ -1,0 +1,242 @@
+"""Host-side mirror of the reference's three custom ops and of its Python glue
+(python/effective_transformer/__init__.py:32-84), on torch-ROCm tensors.
+
+torch is used for device memory and the current stream only; all computation happens in
+libet_hip.so through the C ABI.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+
+_handles: Dict[int, C.c_void_p] = {}
+_workspaces: Dict[Tuple[int, str], torch.Tensor] = {}
+_lock = threading.Lock()
+
+
+def _dtype_code(t: torch.dtype) -> int:
+    if t == torch.float32:
+        return _lib.ET_FP32
+    if t == torch.float16:
+        return _lib.ET_FP16
+    raise TypeError("only float32 and float16 tensors are supported, got %s" % t)
+
+
+def handle(device: torch.device) -> C.c_void_p:
+    """One library handle per GPU."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    with _lock:
+        h = _handles.get(idx)
+        if h is None:
+            h = C.c_void_p()
+            _lib.check(_lib.load().et_create(C.byref(h), idx), None)
+            _handles[idx] = h
+        return h
+
+
+def _workspace(device: torch.device, kind: str, nbytes: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), kind)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise ValueError("tensors must live on the GPU")
+        if not t.is_contiguous():
+            raise ValueError("tensors must be contiguous")
+
+
+# --------------------------------------------------------------------------- the three ops
+
+def effective_transformer_input(from_tensor: torch.Tensor, mask: torch.Tensor, batch_size: int, from_seq_len: int,
+                                to_seq_len: int, head_num: int, size_per_head: int, return_host_count: bool = False):
+    """EffectiveTransformerInput (tf_op/bert_transformer_op.cc:249-340): returns
+    (to_tensor, valid_word_num, batch_idx, word_idx) with the shapes of the reference op; the
+    batch is taken from from_tensor.shape[0] ("dynamic batch size").  With
+    return_host_count=True the valid-token count is also returned as a Python int (one
+    stream synchronisation, as in the reference)."""
+    lib = _lib.load()
+    _require_cuda(from_tensor, mask)
+    if mask.dtype != torch.int32:
+        raise TypeError("mask must be int32")
+    B = from_tensor.shape[0]
+    S = from_seq_len
+    dev = from_tensor.device
+    to_tensor = torch.empty_like(from_tensor)
+    valid_word_num = torch.empty(1, dtype=torch.int32, device=dev)
+    batch_idx = torch.empty_like(mask)
+    word_idx = torch.empty_like(mask)
+    nbytes = lib.et_input_workspace_bytes(B, S)
+    ws = _workspace(dev, "input", nbytes)
+    host = C.c_int32(-1)
+    h = handle(dev)
+    st = lib.et_input(h, _dtype_code(from_tensor.dtype), _p(from_tensor), _p(mask), _p(to_tensor), _p(valid_word_num),
+                      _p(batch_idx), _p(word_idx), B, S, head_num, size_per_head, _p(ws), ws.numel(), _stream(),
+                      C.byref(host) if return_host_count else None)
+    _lib.check(st, h)
+    if return_host_count:
+        return to_tensor, valid_word_num, batch_idx, word_idx, int(host.value)
+    return to_tensor, valid_word_num, batch_idx, word_idx
+
+
+class LayerWeights:
+    """The 16 tensors of one layer on the device, keyed by the attribute names of the
+    reference op (tf_op/bert_transformer_op.cc:44-77)."""
+
+    ATTRS = ("attr_kernel_q", "attr_kernel_k", "attr_kernel_v", "attr_bias_q", "attr_bias_k", "attr_bias_v",
+             "attr_output_kernel", "attr_output_bias", "attr_output_layernorm_beta", "attr_output_layernorm_gamma",
+             "inter_kernel", "inter_bias", "output_kernel", "output_bias", "output_layernorm_beta",
+             "output_layernorm_gamma")
+
+    def __init__(self, device, dtype: torch.dtype, **tensors):
+        missing = [a for a in self.ATTRS if a not in tensors]
+        if missing:
+            raise ValueError("missing weights: %s" % missing)
+        self.t = {}
+        for a in self.ATTRS:
+            v = tensors[a]
+            if isinstance(v, np.ndarray):
+                v = torch.from_numpy(np.ascontiguousarray(v))
+            self.t[a] = v.to(device=device, dtype=dtype).contiguous()
+        s = _lib.LayerWeights()
+        s.attr_kernel_Q = self.t["attr_kernel_q"].data_ptr()
+        s.attr_kernel_K = self.t["attr_kernel_k"].data_ptr()
+        s.attr_kernel_V = self.t["attr_kernel_v"].data_ptr()
+        s.attr_bias_Q = self.t["attr_bias_q"].data_ptr()
+        s.attr_bias_K = self.t["attr_bias_k"].data_ptr()
+        s.attr_bias_V = self.t["attr_bias_v"].data_ptr()
+        for name in ("attr_output_kernel", "attr_output_bias", "attr_output_layernorm_gamma",
+                     "attr_output_layernorm_beta", "inter_kernel", "inter_bias", "output_kernel", "output_bias",
+                     "output_layernorm_gamma", "output_layernorm_beta"):
+            setattr(s, name, self.t[name].data_ptr())
+        self.struct = s
+
+    @classmethod
+    def from_slots(cls, device, dtype, slots: Sequence):
+        """slots: the 16 arrays of one layer in the order of the reference's `weights_value`
+        (python/effective_transformer/__init__.py:55-74):
+        q_k,q_b,k_k,k_b,v_k,v_b,ao_k,ao_b,ao_ln_beta,ao_ln_gamma,i_k,i_b,o_k,o_b,o_ln_beta,o_ln_gamma."""
+        if len(slots) != 16:
+            raise ValueError("a layer has 16 weight tensors")
+        return cls(device, dtype,
+                   attr_kernel_q=slots[0], attr_bias_q=slots[1], attr_kernel_k=slots[2], attr_bias_k=slots[3],
+                   attr_kernel_v=slots[4], attr_bias_v=slots[5], attr_output_kernel=slots[6],
+                   attr_output_bias=slots[7], attr_output_layernorm_beta=slots[8],
+                   attr_output_layernorm_gamma=slots[9], inter_kernel=slots[10], inter_bias=slots[11],
+                   output_kernel=slots[12], output_bias=slots[13], output_layernorm_beta=slots[14],
+                   output_layernorm_gamma=slots[15])
+
+
+def effective_transformer(from_tensor: torch.Tensor, to_tensor: torch.Tensor, attr_mask: torch.Tensor,
+                          valid_word_num: torch.Tensor, batch_idx: torch.Tensor, word_idx: torch.Tensor,
+                          weights: LayerWeights, batch_size: int, from_seq_len: int, to_seq_len: int, head_num: int,
+                          size_per_head: int, valid_word_num_hint: int = -1,
+                          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """EffectiveTransformer layer op (tf_op/bert_transformer_op.cc:44-77, 180-221).  Output has
+    the shape of from_tensor; rows beyond the valid-token count are left as allocated."""
+    lib = _lib.load()
+    _require_cuda(from_tensor, to_tensor, attr_mask, valid_word_num, batch_idx, word_idx)
+    B = from_tensor.shape[0]
+    dev = from_tensor.device
+    if attr_mask.dtype != from_tensor.dtype:
+        raise TypeError("attr_mask must have the dtype of from_tensor")
+    if out is None:
+        out = torch.empty_like(from_tensor)
+    code = _dtype_code(from_tensor.dtype)
+    nbytes = lib.et_layer_workspace_bytes(code, B, from_seq_len, head_num, size_per_head)
+    ws = _workspace(dev, "layer", nbytes)
+    h = handle(dev)
+    st = lib.et_layer(h, code, C.byref(weights.struct), _p(from_tensor), _p(to_tensor), _p(attr_mask),
+                      _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B, from_seq_len, to_seq_len, head_num,
+                      size_per_head, valid_word_num_hint, _p(ws), ws.numel(), _stream())
+    _lib.check(st, h)
+    return out
+
+
+def effective_transformer_output(from_tensor: torch.Tensor, valid_word_num: torch.Tensor, batch_idx: torch.Tensor,
+                                 word_idx: torch.Tensor, batch_size: int, from_seq_len: int, to_seq_len: int,
+                                 head_num: int, size_per_head: int) -> torch.Tensor:
+    """EffectiveTransformerOutput (tf_op/bert_transformer_op.cc:359-431): [B,S,H] with zeros at
+    padding."""
+    lib = _lib.load()
+    _require_cuda(from_tensor, valid_word_num, batch_idx, word_idx)
+    B = from_tensor.shape[0]
+    to_tensor = torch.empty_like(from_tensor)
+    h = handle(from_tensor.device)
+    st = lib.et_output(h, _dtype_code(from_tensor.dtype), _p(from_tensor), _p(valid_word_num), _p(batch_idx),
+                       _p(word_idx), _p(to_tensor), B, from_seq_len, head_num, size_per_head, _stream())
+    _lib.check(st, h)
+    return to_tensor
+
+
+# --------------------------------------------------------------------------- the glue
+
+class EffectiveTransformerEncoder:
+    """Input -> L x Layer -> Output with the weights resident on the device (the reference bakes
+    them into op attributes at graph build, python/effective_transformer/__init__.py:48-76)."""
+
+    def __init__(self, num_layers: int, head_num: int, size_per_head: int, weights_value: Sequence, dtype: torch.dtype,
+                 device="cuda"):
+        if len(weights_value) != 16 * num_layers:
+            raise ValueError("expected %d weight tensors, got %d" % (16 * num_layers, len(weights_value)))
+        self.device = torch.device(device)
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
+        self.dtype = dtype
+        self.head_num, self.size_per_head, self.num_layers = head_num, size_per_head, num_layers
+        self.layers: List[LayerWeights] = [
+            LayerWeights.from_slots(self.device, dtype, weights_value[16 * l:16 * l + 16]) for l in range(num_layers)]
+        self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor]] = {}
+
+    def __call__(self, from_tensor: torch.Tensor, input_mask: torch.Tensor, attention_mask: torch.Tensor,
+                 sync_count: bool = True) -> torch.Tensor:
+        B, S = input_mask.shape
+        hn, d = self.head_num, self.size_per_head
+        if sync_count:
+            x, vwn, bidx, widx, T = effective_transformer_input(from_tensor, input_mask, B, S, S, hn, d,
+                                                                return_host_count=True)
+        else:
+            x, vwn, bidx, widx = effective_transformer_input(from_tensor, input_mask, B, S, S, hn, d)
+            T = -1
+        key = tuple(from_tensor.shape)
+        bufs = self._bufs.get(key)
+        if bufs is None:
+            bufs = (torch.empty_like(from_tensor), torch.empty_like(from_tensor))
+            self._bufs[key] = bufs
+        for l, w in enumerate(self.layers):
+            out = bufs[l & 1]
+            effective_transformer(x, x, attention_mask, vwn, bidx, widx, w, B, S, S, hn, d, valid_word_num_hint=T,
+                                  out=out)
+            x = out
+        return effective_transformer_output(x, vwn, bidx, widx, B, S, S, hn, d)
+
+
+def get_sequence_output(config, max_batch_size, max_seq_length, attention_mask, input_mask, from_tensor,
+                        weights_value):
+    """Same argument list as the reference's get_sequence_output
+    (python/effective_transformer/__init__.py:32-35).  `config` needs num_attention_heads,
+    hidden_size and num_hidden_layers."""
+    head_num = config.num_attention_heads
+    size_per_head = int(config.hidden_size / config.num_attention_heads)
+    enc = EffectiveTransformerEncoder(config.num_hidden_layers, head_num, size_per_head, weights_value,
+                                      from_tensor.dtype, from_tensor.device)
+    return enc(from_tensor, input_mask, attention_mask)

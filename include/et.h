@@ -1,0 +1,199 @@
+/*
+ * et.h -- C ABI of the MI355X (gfx950) padding-free BERT encoder library, libet_hip.so.
+ *
+ * The entry points replace, one for one, the GPU functors behind the three TensorFlow ops
+ * of bytedance/effective_transformer and the kernel launchers those functors call.  Paths
+ * in the comments are relative to the reference tree.
+ *
+ * Conventions
+ *   - extern "C", plain pointers and sizes, POD structs; no exception crosses the boundary.
+ *   - Every pointer named *_dev / every tensor argument is DEVICE memory owned by the caller
+ *     (inputs, outputs, weights and workspace).  No entry point allocates or frees device
+ *     memory.
+ *   - Every call returns an et_status; et_last_error() gives the message of the last failure
+ *     on that handle (replaces the reference's std::runtime_error -> errors::Internal path,
+ *     common.h:73-81, tf_op/bert_transformer_op.cu.cc:251-258).
+ *   - Work is enqueued on the hipStream_t passed as `stream` (an opaque void* here) and is
+ *     asynchronous unless a host output (valid_word_num_host) is requested.
+ *   - Dense kernels are [in,out] row-major, biases / gamma / beta are [out]
+ *     (tf_op/bert_transformer_op.cu.cc:110-119).
+ *   - One handle may be used from several threads: calls on it are serialised by an
+ *     internal mutex (the reference's cublas_mutex_, tf_op/bert_transformer_op.cc:213).
+ */
+#ifndef ET_H_
+#define ET_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum et_status {
+  ET_OK = 0,
+  ET_INVALID_ARGUMENT = 1,    /* null pointer, bad dimension, from_seq_len != to_seq_len ... */
+  ET_WORKSPACE_TOO_SMALL = 2,
+  ET_UNSUPPORTED = 3,         /* shape outside what the kernels are built for */
+  ET_LAUNCH_FAILURE = 4,      /* hipGetLastError() after a launch */
+  ET_RUNTIME_ERROR = 5        /* any other HIP runtime error */
+} et_status;
+
+/* OperationType{FP32,HALF}, common.h:26 */
+typedef enum et_dtype { ET_FP32 = 0, ET_FP16 = 1 } et_dtype;
+
+typedef struct et_context* et_handle;
+
+/* Handle life cycle.  Replaces the per-op state created in the OpKernel constructors
+ * (cublasCreate at tf_op/bert_transformer_op.cc:171).  `device` is a HIP device ordinal. */
+et_status et_create(et_handle* out, int device);
+et_status et_destroy(et_handle h);
+/* Message of the last failing call on `h` (or of the last failing et_create on this thread
+ * when h is NULL).  Never NULL. */
+const char* et_last_error(et_handle h);
+const char* et_status_string(et_status s);
+/* 1 when the library was built for the architecture of `device` and a kernel runs there. */
+int et_device_ok(int device);
+
+/* The 16 per-layer tensors, named as the fields of EncoderInitParam<T>
+ * (tf_op/bert_transformer_op.h:66-96).  All device pointers of the layer's dtype. */
+typedef struct et_layer_weights {
+  const void* attr_kernel_Q;               /* [H,H]  */
+  const void* attr_kernel_K;               /* [H,H]  */
+  const void* attr_kernel_V;               /* [H,H]  */
+  const void* attr_bias_Q;                 /* [H]    */
+  const void* attr_bias_K;                 /* [H]    */
+  const void* attr_bias_V;                 /* [H]    */
+  const void* attr_output_kernel;          /* [H,H]  */
+  const void* attr_output_bias;            /* [H]    */
+  const void* attr_output_layernorm_gamma; /* [H]    */
+  const void* attr_output_layernorm_beta;  /* [H]    */
+  const void* inter_kernel;                /* [H,4H] */
+  const void* inter_bias;                  /* [4H]   */
+  const void* output_kernel;               /* [4H,H] */
+  const void* output_bias;                 /* [H]    */
+  const void* output_layernorm_gamma;      /* [H]    */
+  const void* output_layernorm_beta;       /* [H]    */
+} et_layer_weights;
+
+/* Workspace sizes in bytes (sized by element type; the reference sizes its layer buffer in
+ * bytes but indexes it in elements, tf_op/bert_transformer_op.cu.cc:75-96). */
+size_t et_input_workspace_bytes(int batch_size, int seq_len);
+size_t et_layer_workspace_bytes(et_dtype dtype, int batch_size, int seq_len, int head_num, int size_per_head);
+/* scratch for the per-sequence start table some kernel-level entry points build */
+size_t et_seq_workspace_bytes(int batch_size);
+
+/* ---- the three ops ------------------------------------------------------------------ */
+
+/* EffectiveTransformerInputOpFunctor::Compute, tf_op/bert_transformer_op.cu.cc:266-331
+ * (op registered at tf_op/bert_transformer_op.cc:249-274).
+ *   from_tensor [B,S,H], mask int32 [B,S] (0/1)  ->
+ *   to_tensor (first T rows of [B*S,H] defined), valid_word_num_dev int32[1],
+ *   batch_idx / word_idx int32[B*S] (first T defined).
+ * valid_word_num_host: optional; when non-NULL the call synchronises the stream and stores T
+ * there (the reference always synchronises, :306-310). */
+et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask,
+                   void* to_tensor, int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx,
+                   int batch_size, int seq_len, int head_num, int size_per_head,
+                   void* workspace, size_t workspace_bytes, void* stream, int32_t* valid_word_num_host);
+
+/* EffectiveTransformerOpFunctor::Compute, tf_op/bert_transformer_op.cu.cc:33-260
+ * (op registered at tf_op/bert_transformer_op.cc:44-77): one encoder layer on packed tokens.
+ *   from_tensor, to_tensor [T,H] packed; attr_mask [B,S,S] of dtype (1 = attend);
+ *   out [T,H] packed (rows >= T untouched).
+ * valid_word_num_hint: T when the host knows it (grids are sized exactly), or -1: grids are
+ * then sized for B*S rows and every kernel bounds itself by *valid_word_num_dev, so the call
+ * never blocks the host (the reference copies T back every layer, :99-101).
+ * from_seq_len must equal to_seq_len (tf_op/bert_transformer_op.cc:130-131).  `out` must not
+ * alias from_tensor/to_tensor. */
+et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
+                   const void* from_tensor, const void* to_tensor, const void* attr_mask,
+                   const int32_t* valid_word_num_dev, const int32_t* batch_idx, const int32_t* word_idx,
+                   void* out, int batch_size, int from_seq_len, int to_seq_len, int head_num, int size_per_head,
+                   int valid_word_num_hint, void* workspace, size_t workspace_bytes, void* stream);
+
+/* EffectiveTransformerOutputOpFunctor::Compute, tf_op/bert_transformer_op.cu.cc:339-373
+ * (op registered at tf_op/bert_transformer_op.cc:359-380): to_tensor [B,S,H] = 0 at padding,
+ * from_tensor row t at (batch_idx[t], word_idx[t]).  batch_idx/word_idx must be those written
+ * by et_input (ascending in b*S+s). */
+et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* valid_word_num_dev,
+                    const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor,
+                    int batch_size, int seq_len, int head_num, int size_per_head, void* stream);
+
+/* ---- kernel-level entry points (unit tests, profiling in isolation) ----------------- */
+
+/* exclusiveScan_kernelLauncher, cuda/cuda_kernels.h:29 (cuda/cuda_kernels.cu:709-718).
+ * workspace: et_input_workspace_bytes(1, length). */
+et_status et_exclusive_scan(et_handle h, int32_t* d_out, const int32_t* d_in, int length,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* compressBertInput_kernelLauncher, cuda/cuda_kernels.h:31-35 (cuda/cuda_kernels.cu:278-384). */
+et_status et_compress(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask,
+                      const int32_t* prefix_sum, void* to_tensor, int32_t* batch_idx, int32_t* word_idx,
+                      int batch_size, int seq_len, int hidden_dim, void* stream);
+
+/* restoreBertOutput_kernelLauncher, cuda/cuda_kernels.h:37-41 (cuda/cuda_kernels.cu:389-468),
+ * fused with the zero fill the output op does first (tf_op/bert_transformer_op.cu.cc:354-355). */
+et_status et_restore(et_handle h, et_dtype dtype, void* to_tensor, const void* from_tensor,
+                     const int32_t* batch_idx, const int32_t* word_idx, const int32_t* valid_word_num_dev,
+                     int batch_size, int seq_len, int hidden_dim, void* stream);
+
+/* add_bias_act_kernelLauncher, cuda/cuda_kernels.h:22-23 (cuda/cuda_kernels.cu:88-150):
+ * out[m,n] = gelu_tanh(out + bias), in place.  m_dev (optional) bounds the rows on the device. */
+et_status et_add_bias_act(et_handle h, et_dtype dtype, void* out, const void* bias, int m, int n,
+                          const int32_t* m_dev, void* stream);
+
+/* add_bias_input_layernorm_kernelLauncher, cuda/cuda_kernels.h:25-27 (cuda/cuda_kernels.cu:157-271):
+ * out[m,n] = LayerNorm(out + input + bias) * gamma + beta, eps 1e-6, in place. */
+et_status et_add_bias_input_layernorm(et_handle h, et_dtype dtype, void* out, const void* input,
+                                      const void* bias, const void* gamma, const void* beta,
+                                      int m, int n, const int32_t* m_dev, void* stream);
+
+/* add_QKV_bias_padding_kernelLauncher, cuda/attention.h:25-35 (cuda/attention.cu:105-242), fused
+ * with the zero fill that precedes it (tf_op/bert_transformer_op.cu.cc:146):
+ * q/k/v_buf [B,heads,S,d] = 0 at padding, src[t] + bias at (batch_idx[t], :, word_idx[t], :).
+ * workspace: et_seq_workspace_bytes(B). */
+et_status et_add_qkv_bias_padding(et_handle h, et_dtype dtype,
+                                  const void* Q, const void* bias_Q, const void* K, const void* bias_K,
+                                  const void* V, const void* bias_V, void* q_buf, void* k_buf, void* v_buf,
+                                  const int32_t* valid_word_num_dev, int batch_size, int seq_len,
+                                  int head_num, int size_per_head,
+                                  const int32_t* batch_idx, const int32_t* word_idx,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* softmax_kernel_kernelLauncher, cuda/attention.h:37-42 (cuda/attention.cu:249-382): in-place
+ * masked, scaled softmax of qk_buf [B,heads,S,S] with attr_mask [B,S,S]. */
+et_status et_softmax(et_handle h, et_dtype dtype, void* qk_buf, const void* attr_mask,
+                     int batch_size, int head_num, int seq_len, float scaler, void* stream);
+
+/* transpose_rm_padding_kernelLauncher, cuda/attention.h:44-51 (cuda/attention.cu:387-492):
+ * src [B,heads,S,d] -> dst packed [T,heads*d]. */
+et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, void* dst,
+                                  const int32_t* valid_word_num_dev, int batch_size, int seq_len,
+                                  int head_num, int size_per_head,
+                                  const int32_t* batch_idx, const int32_t* word_idx, void* stream);
+
+/* The attention block of the layer in one kernel: batched QK^T, masked softmax, batched PV and
+ * un-padding (tf_op/bert_transformer_op.cu.cc:159-192).
+ *   qkv_layout 0: q/k/v are the padded [B,heads,S,d] buffers add_QKV_bias_padding writes;
+ *   qkv_layout 1: q/k/v point into packed token-major rows (row t, column head*d + j) with row
+ *                 stride `packed_ld` elements (bias already added).
+ *   dst packed [T,heads*d].  workspace: et_seq_workspace_bytes(B). */
+et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v, int qkv_layout,
+                       int packed_ld, const void* attr_mask, void* dst,
+                       const int32_t* valid_word_num_dev, int batch_size, int seq_len,
+                       int head_num, int size_per_head,
+                       const int32_t* batch_idx, const int32_t* word_idx,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* Replaces the cublasGemmEx call sites (tf_op/bert_transformer_op.cu.cc:110-141, 200-240):
+ * C[m,n] = A[m,k] . B[k,n], all row-major, alpha = 1, beta = 0, fp32 accumulation, C of dtype.
+ * bias (optional, [n]) is added to the rounded product (in the element type, as the reference's
+ * following kernel would).  m_dev (optional) bounds the rows on the device. */
+et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias,
+                  int m, int n, int k, const int32_t* m_dev, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ET_H_ */

@@ -1,0 +1,61 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol include/et.h declares,
+and its host-only entry points (sizes, status strings, argument errors) behave.  No kernel runs."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from effective_transformer_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "et.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(et_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
+
+
+def test_status_strings_and_sizes():
+    lib = _lib.load()
+    assert lib.et_status_string(0) == b"ET_OK"
+    assert lib.et_status_string(2) == b"ET_WORKSPACE_TOO_SMALL"
+    assert lib.et_input_workspace_bytes(1000, 64) >= 4 * 63
+    assert lib.et_input_workspace_bytes(0, 64) == 0
+    # the layer workspace is sized by element type (the reference sizes in bytes and indexes in elements)
+    h16 = lib.et_layer_workspace_bytes(_lib.ET_FP16, 500, 64, 12, 64)
+    h32 = lib.et_layer_workspace_bytes(_lib.ET_FP32, 500, 64, 12, 64)
+    assert h32 > 1.9 * h16 > 0
+    rows, H = 500 * 64, 768
+    assert h16 >= rows * 9 * H * 2
+    assert lib.et_seq_workspace_bytes(256) >= 257 * 4
+
+
+def test_null_handle_and_create_without_gpu():
+    lib = _lib.load()
+    assert lib.et_input(None, 0, None, None, None, None, None, None, 1, 1, 1, 1, None, 0, None, None) == 1
+    assert b"null handle" in lib.et_last_error(None)
+    import torch
+    if not torch.cuda.is_available():
+        h = C.c_void_p()
+        st = lib.et_create(C.byref(h), 0)
+        assert st != 0 and not h.value
+        assert lib.et_last_error(None).startswith(b"[ET][ERROR]")
+    assert lib.et_destroy(None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(ImportError):
+        _lib.load()

@@ -1,0 +1,138 @@
+"""Parity of the three ops (Input -> L x Layer -> Output through the C ABI) against the CPU
+oracle on the seeded workloads, plus size-independent properties at the full benchmark sizes."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import et_oracle as o
+from gpu_util import TDT, dev, run_encoder, subset_workload
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(w, layers=None):
+    wl = w["wl"]
+    weights = w["weights"] if layers is None else w["weights"][:16 * layers]
+    return o.encoder(w["x"], w["mask"], w["attr_mask"], weights, wl.heads, wl.d, wl.dtype)
+
+
+def _check(got, want, mask, dtype):
+    valid = mask.astype(bool)
+    assert np.all(got[~valid] == 0)                              # the Output op zero-fills padding
+    g, w_ = got[valid].astype(np.float64), want[valid].astype(np.float64)
+    if dtype == "fp32":
+        # fp32 bar: 1e-4 relative (LayerNorm outputs are O(1); relative to max(|want|, 1))
+        err = np.abs(g - w_) / np.maximum(np.abs(w_), 1.0)
+        assert err.max() < 1e-4, err.max()
+    else:
+        # fp16 bar: 2e-2 max-abs after 12 layers
+        assert np.abs(g - w_).max() < 2e-2, np.abs(g - w_).max()
+    return np.abs(g - w_).max()
+
+
+@pytest.mark.parametrize("random_affine", [False, True])
+def test_cfg1_single_layer_fp32(random_affine):
+    w = o.make_workload("cfg1", random_affine=random_affine)
+    got = run_encoder(w)
+    print("cfg1 max abs diff", _check(got, _oracle(w), w["mask"], "fp32"), flush=True)
+    # and the reference's own check: agreement with the standard BERT graph on valid tokens
+    std = o.tf_graph_encoder(w["x"], w["attr_mask"], w["weights"], w["wl"].heads, w["wl"].d)
+    valid = w["mask"].astype(bool)
+    assert np.abs(got[valid] - std[valid]).max() < 1e-4
+
+
+def test_cfg1_fp16_variant():
+    w = o.make_workload("cfg1", random_affine=True)
+    w16 = dict(w, wl=o.Workload(**{**w["wl"].__dict__, "dtype": "fp16"}), x=w["x"].astype(np.float16),
+               attr_mask=w["attr_mask"].astype(np.float16), weights=[a.astype(np.float16) for a in w["weights"]])
+    got = run_encoder(w16)
+    print("cfg1/fp16 max abs diff", _check(got, _oracle(w16), w16["mask"], "fp16"), flush=True)
+
+
+def test_cfg2_twelve_layers_fp16():
+    w = o.make_workload("cfg2")
+    got = run_encoder(w)
+    print("cfg2 max abs diff", _check(got, _oracle(w), w["mask"], "fp16"), flush=True)
+    # device-side token count (no host hint) gives the same bits
+    got2 = run_encoder(w, hint=False)
+    assert np.array_equal(got, got2)
+
+
+def test_cfg2_random_affine_fp32_twelve_layers():
+    w = o.make_workload("cfg2", random_affine=True)
+    w32 = dict(w, wl=o.Workload(**{**w["wl"].__dict__, "dtype": "fp32"}), x=w["x"].astype(np.float32),
+               attr_mask=w["attr_mask"].astype(np.float32), weights=[a.astype(np.float32) for a in w["weights"]])
+    sub = subset_workload(w32, np.arange(24))
+    got = run_encoder(sub)
+    print("cfg2/fp32 12 layers max abs diff", _check(got, _oracle(sub), sub["mask"], "fp32"), flush=True)
+
+
+@pytest.mark.parametrize("name,nsub,layers", [("cfg3", 24, 12), ("cfg4", 12, 12), ("cfg5", 8, 24)])
+def test_full_size_properties_and_subset_oracle(name, nsub, layers):
+    """At the benchmark sizes the oracle is too slow, so: (1) sequences are independent, hence a
+    run on a subset of the sequences must reproduce the full run's rows bit for bit, and the
+    subset is small enough for the oracle; (2) permuting the batch permutes the output;
+    (3) padding is zero."""
+    print("full-size", name, flush=True)
+    w = o.make_workload(name)
+    wl = w["wl"]
+    full = run_encoder(w)
+    assert np.all(full[~w["mask"].astype(bool)] == 0)
+    assert np.isfinite(full.astype(np.float32)).all()
+    rng = np.random.RandomState(1)
+    idx = np.sort(rng.choice(wl.B, nsub, replace=False))
+    sub = subset_workload(w, idx)
+    got_sub = run_encoder(sub)
+    assert np.array_equal(got_sub, full[idx])
+    print(name, "subset max abs diff vs oracle", _check(got_sub, _oracle(sub), sub["mask"], wl.dtype), flush=True)
+    perm = rng.permutation(wl.B)
+    wp = subset_workload(w, perm)
+    assert np.array_equal(run_encoder(wp), full[perm])
+
+
+def test_empty_batch_of_tokens_and_holes():
+    w = o.make_workload("cfg1", random_affine=True)
+    wl = w["wl"]
+    zero = dict(w, mask=np.zeros_like(w["mask"]), attr_mask=np.zeros_like(w["attr_mask"]))
+    out = run_encoder(zero)
+    assert np.all(out == 0)
+    out = run_encoder(zero, hint=False)
+    assert np.all(out == 0)
+    # a mask with holes and an attention mask that is not tied to it
+    rng = np.random.RandomState(5)
+    mask = (rng.random_sample(w["mask"].shape) < 0.6).astype(np.int32)
+    attr = (rng.random_sample(w["attr_mask"].shape) < 0.8).astype(np.float32)
+    hol = dict(w, mask=mask, attr_mask=attr)
+    got = run_encoder(hol)
+    print("holes max abs diff", _check(got, _oracle(hol), mask, "fp32"), flush=True)
+
+
+def test_error_paths():
+    from effective_transformer_amd import _lib, ops
+    lib = _lib.load()
+    h = ops.handle(torch.device("cuda", 0))
+    w = o.make_workload("cfg1")
+    wl = w["wl"]
+    x = dev(w["x"]); mask = dev(w["mask"]); attr = dev(w["attr_mask"])
+    to, vwn, bidx, widx = ops.effective_transformer_input(x, mask, wl.B, wl.S, wl.S, wl.heads, wl.d)
+    lw = ops.LayerWeights.from_slots(x.device, torch.float32, w["weights"][:16])
+    with pytest.raises(_lib.EtError) as e:       # from_seq_len != to_seq_len
+        ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S + 1, wl.heads, wl.d)
+    assert e.value.status == 1 and "from_seq_len == to_seq_len" in str(e.value)
+    with pytest.raises(_lib.EtError) as e:       # size_per_head the attention kernel is not built for
+        ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S, wl.heads * 2, wl.d // 2)
+    assert e.value.status == 3
+    out = torch.empty_like(to)
+    st = lib.et_layer(h, 0, C.byref(lw.struct), to.data_ptr(), to.data_ptr(), attr.data_ptr(), vwn.data_ptr(),
+                      bidx.data_ptr(), widx.data_ptr(), out.data_ptr(), wl.B, wl.S, wl.S, wl.heads, wl.d, -1,
+                      out.data_ptr(), 1024, None)
+    assert st == 2 and b"ET_WORKSPACE_TOO_SMALL" in lib.et_last_error(h)
+    st = lib.et_layer(h, 0, C.byref(lw.struct), to.data_ptr(), to.data_ptr(), attr.data_ptr(), vwn.data_ptr(),
+                      bidx.data_ptr(), widx.data_ptr(), to.data_ptr(), wl.B, wl.S, wl.S, wl.heads, wl.d, -1,
+                      out.data_ptr(), 1 << 30, None)
+    assert st == 1 and b"alias" in lib.et_last_error(h)
+    with pytest.raises(TypeError):
+        ops.effective_transformer_input(x.to(torch.bfloat16), mask, wl.B, wl.S, wl.S, wl.heads, wl.d)
+    torch.cuda.synchronize()

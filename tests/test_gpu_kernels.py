@@ -1,0 +1,296 @@
+"""Parity of every kernel-level entry point of the C ABI against the CPU oracle, on a real
+MI355X.  Integer/byte work is bit-exact; floating point carries the tolerance written at each
+assertion."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import et_oracle as o
+from gpu_util import TDT, assert_half_close, dev, half_ulp
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def k():
+    from effective_transformer_amd import kernel_ops
+    return kernel_ops
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from effective_transformer_amd import ops
+    return ops
+
+
+# ---------------------------------------------------------------------------- scan ---
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 2048 + 17, 64000, (1 << 20) + 3,
+                               1100 * 1024 + 5])
+def test_exclusive_scan(k, n):
+    print("scan n=%d" % n, flush=True)
+    rng = np.random.RandomState(n % 1000)
+    for kind in ("mask", "ints"):
+        a = (rng.random_sample(n) < 0.63).astype(np.int32) if kind == "mask" else rng.randint(0, 50, n).astype(np.int32)
+        got = k.exclusive_scan(dev(a)).cpu().numpy()
+        assert np.array_equal(got, o.exclusive_scan(a)), kind
+
+
+def _input_case(ops, x, mask, dtype):
+    B, S, H = x.shape
+    heads = H // 64 if H % 64 == 0 else 1
+    d = H // heads
+    to, vwn, bidx, widx, T = ops.effective_transformer_input(dev(x, TDT[dtype]), dev(mask), B, S, S, heads, d,
+                                                             return_host_count=True)
+    wto, wT, wb, ww, _ = o.input_op_fast(o.rnd(x, dtype), mask)
+    assert T == wT == int(vwn.item())
+    assert np.array_equal(bidx.cpu().numpy().reshape(-1)[:T], wb)
+    assert np.array_equal(widx.cpu().numpy().reshape(-1)[:T], ww)
+    got = to.cpu().numpy().reshape(B * S, H)[:T]
+    assert np.array_equal(got.view(np.uint8), wto.view(np.uint8))
+    return to, vwn, bidx, widx, T
+
+
+def test_input_known_answers(ops):
+    ka = json.load(open(os.path.join(GOLD, "known_answers.json")))
+    fig = np.array(ka["figure_4x8"]["mask"], dtype=np.int32)
+    x = np.random.RandomState(0).randn(4, 8, 64).astype(np.float32)
+    to, vwn, bidx, widx, T = _input_case(ops, x, fig, "fp32")
+    assert T == ka["figure_4x8"]["valid_word_num"]
+    padded = (bidx.cpu().numpy().reshape(-1)[:T].astype(np.int64) * 8 + widx.cpu().numpy().reshape(-1)[:T])
+    assert padded[:8].tolist() == ka["figure_4x8"]["packed_to_padded_first8"]
+    rd = np.array(ka["readme_3x5"]["mask"], dtype=np.int32)
+    tok = np.zeros((3, 5, 8), np.float16)
+    tok[..., 0] = np.array(ka["readme_3x5"]["tokens_padded"])
+    to, vwn, bidx, widx, T = _input_case(ops, tok, rd, "fp16")
+    assert T == 7 and to.cpu().numpy().reshape(15, 8)[:7, 0].tolist() == ka["readme_3x5"]["tokens_packed"]
+
+
+@pytest.mark.parametrize("case", ["holes", "ones", "zeros", "last0", "last1", "single"])
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_input_edge_masks(ops, k, case, dtype):
+    print("input edge", case, dtype, flush=True)
+    rng = np.random.RandomState(len(case))
+    B, S, H = 37, 29, 128
+    mask = (rng.random_sample((B, S)) < 0.55).astype(np.int32)
+    if case == "ones":
+        mask[:] = 1
+    elif case == "zeros":
+        mask[:] = 0
+    elif case == "last0":
+        mask[-1, -1] = 0
+    elif case == "last1":
+        mask[-1, -1] = 1
+    elif case == "single":
+        B, S = 1, 1
+        mask = np.ones((1, 1), np.int32)
+    x = rng.randn(B, S, H).astype(np.float32)
+    to, vwn, bidx, widx, T = _input_case(ops, x, mask, dtype)
+    # Output op: zero at padding, original rows elsewhere (round trip)
+    back = ops.effective_transformer_output(to, vwn, bidx, widx, B, S, S, 2, H // 2).cpu().numpy()
+    want = o.rnd(x, dtype) * mask[..., None].astype(o._np_dtype(dtype))
+    assert np.array_equal(back, want)
+
+
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+def test_input_output_on_workload_masks(ops, name):
+    print("input workload", name, flush=True)
+    w = o.make_workload(name, with_inputs=False)
+    wl = w["wl"]
+    rng = np.random.RandomState(7)
+    x = rng.randn(wl.B, wl.S, wl.H).astype(np.float32)
+    to, vwn, bidx, widx, T = _input_case(ops, x, w["mask"], wl.dtype)
+    dig = json.load(open(os.path.join(GOLD, "workload_digests.json")))
+    assert T == dig[name]["T"]
+    back = ops.effective_transformer_output(to, vwn, bidx, widx, wl.B, wl.S, wl.S, wl.heads, wl.d).cpu().numpy()
+    want = o.rnd(x, wl.dtype) * w["mask"][..., None].astype(o._np_dtype(wl.dtype))
+    assert np.array_equal(back, want)
+    # checksum of the packed rows equals the checksum of the valid rows
+    assert np.array_equal(back.astype(np.float64).sum(axis=(0, 1)), want.astype(np.float64).sum(axis=(0, 1)))
+
+
+def test_compress_and_restore_entry_points(k):
+    rng = np.random.RandomState(3)
+    B, S, H = 9, 17, 96
+    mask = (rng.random_sample((B, S)) < 0.5).astype(np.int32)
+    x = rng.randn(B, S, H).astype(np.float16)
+    wto, T, wb, ww, prefix = o.input_op(x, mask)
+    to, bidx, widx = k.compress(dev(x), dev(mask), dev(prefix))
+    assert np.array_equal(to.cpu().numpy().reshape(B * S, H)[:T], wto)
+    assert np.array_equal(bidx.cpu().numpy().reshape(-1)[:T], wb)
+    assert np.array_equal(widx.cpu().numpy().reshape(-1)[:T], ww)
+    vwn = torch.tensor([T], dtype=torch.int32, device="cuda")
+    back = k.restore(to.reshape(B * S, H), bidx, widx, vwn, B, S).cpu().numpy()
+    assert np.array_equal(back, o.restore(wto, T, wb, ww, B, S))
+
+
+# -------------------------------------------------------------------- row kernels ---
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("m,n", [(1, 64), (5, 3072), (134, 3072), (33, 4096), (7, 200)])
+def test_add_bias_act(k, dtype, m, n):
+    print("gelu", dtype, m, n, flush=True)
+    rng = np.random.RandomState(m + n)
+    x = o.rnd(2.5 * rng.randn(m, n), dtype)
+    b = o.rnd(rng.randn(n), dtype)
+    want = o.add_bias_act(x, b, dtype)
+    got = k.add_bias_act(dev(x), dev(b)).cpu().numpy()
+    if dtype == "fp32":
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    else:
+        assert_half_close(got, want, ulps=1.0, frac=0.01, what="gelu")
+    # rows bounded on the device: rows >= *m_dev stay untouched
+    if m > 3:
+        keep = torch.tensor([m - 2], dtype=torch.int32, device="cuda")
+        got2 = k.add_bias_act(dev(x), dev(b), m_dev=keep).cpu().numpy()
+        assert np.array_equal(got2[:m - 2], got[:m - 2]) and np.array_equal(got2[m - 2:], x[m - 2:])
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("m,n", [(1, 768), (134, 768), (50, 1024), (9, 64), (6, 200), (3, 2048)])
+def test_add_bias_input_layernorm(k, dtype, m, n):
+    print("layernorm", dtype, m, n, flush=True)
+    rng = np.random.RandomState(m * 7 + n)
+    out = o.rnd(rng.randn(m, n), dtype)
+    inp = o.rnd(rng.randn(m, n), dtype)
+    bias, gamma, beta = (o.rnd(v, dtype) for v in (0.3 * rng.randn(n), 1 + 0.2 * rng.randn(n), 0.2 * rng.randn(n)))
+    want = o.add_bias_input_layernorm(out, inp, bias, gamma, beta, dtype)
+    got = k.add_bias_input_layernorm(dev(out), dev(inp), dev(bias), dev(gamma), dev(beta)).cpu().numpy()
+    if dtype == "fp32":
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)    # fp32 bar: 1e-4 relative
+    else:
+        assert_half_close(got, want, ulps=1.0, frac=0.01, what="layernorm")
+    if m > 3:
+        keep = torch.tensor([2], dtype=torch.int32, device="cuda")
+        got2 = k.add_bias_input_layernorm(dev(out), dev(inp), dev(bias), dev(gamma), dev(beta), m_dev=keep).cpu().numpy()
+        assert np.array_equal(got2[:2], got[:2]) and np.array_equal(got2[2:], out[2:])
+
+
+# ---------------------------------------------------------------- attention side ---
+
+def _attn_problem(seed, B, S, heads, dtype, holes=False, weird_mask=False):
+    rng = np.random.RandomState(seed)
+    d = 64
+    if holes:
+        mask = (rng.random_sample((B, S)) < 0.6).astype(np.int32)
+        mask[0] = 0                                  # an empty sequence
+        mask[1] = 1
+    else:
+        lens = rng.randint(1, S + 1, size=B)
+        mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.int32)
+    _, T, bi, wi, _ = o.input_op_fast(np.zeros((B, S, 1), np.float32), mask)
+    H = heads * d
+    q, kk, v = (o.rnd(rng.randn(T, H), dtype) for _ in range(3))
+    bq, bk, bv = (o.rnd(0.5 * rng.randn(H), dtype) for _ in range(3))
+    if weird_mask:
+        attr = (rng.random_sample((B, S, S)) < 0.7).astype(np.float32)
+        attr[:, 0, :] = 0                            # fully masked query rows
+    else:
+        attr = np.ascontiguousarray(np.broadcast_to(mask[:, None, :], (B, S, S))).astype(np.float32)
+    return dict(B=B, S=S, heads=heads, d=d, mask=mask, T=T, bi=bi, wi=wi, q=q, k=kk, v=v, bq=bq, bk=bk, bv=bv,
+                attr=o.rnd(attr, dtype))
+
+
+def _idx_dev(p):
+    n = p["B"] * p["S"]
+    bi = np.full(n, -1, np.int32); bi[:p["T"]] = p["bi"]
+    wi = np.full(n, -1, np.int32); wi[:p["T"]] = p["wi"]
+    return dev(bi), dev(wi), torch.tensor([p["T"]], dtype=torch.int32, device="cuda")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("holes", [False, True])
+def test_qkv_bias_padding_and_unpad(k, dtype, holes):
+    p = _attn_problem(11, 6, 13, 3, dtype, holes=holes)
+    bi, wi, vwn = _idx_dev(p)
+    want = o.add_qkv_bias_padding(p["q"], p["bq"], p["k"], p["bk"], p["v"], p["bv"], p["T"], p["B"], p["S"],
+                                  p["heads"], p["d"], p["bi"], p["wi"], dtype)
+    got = k.add_qkv_bias_padding(dev(p["q"]), dev(p["bq"]), dev(p["k"]), dev(p["bk"]), dev(p["v"]), dev(p["bv"]), vwn,
+                                 p["B"], p["S"], p["heads"], p["d"], bi, wi)
+    for g, w_ in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w_)          # one correctly rounded add per element: bit-exact
+    un = k.transpose_rm_padding(got[0], vwn, bi, wi).cpu().numpy()
+    assert np.array_equal(un[:p["T"]], o.transpose_rm_padding(want[0], p["T"], p["bi"], p["wi"]))
+    assert np.all(un[p["T"]:] == 0)                          # rows beyond T untouched
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("S", [1, 7, 32, 64, 100, 128, 300])
+def test_softmax(k, dtype, S):
+    rng = np.random.RandomState(S)
+    B, heads = 3, 2
+    qk = o.rnd(6 * rng.randn(B, heads, S, S), dtype)
+    attr = (rng.random_sample((B, S, S)) < 0.7).astype(np.float32)
+    attr[0, 0] = 0
+    attr = o.rnd(attr, dtype)
+    want = o.softmax(qk, attr, 0.125, dtype)
+    got = k.softmax(dev(qk), dev(attr), 0.125).cpu().numpy()
+    if dtype == "fp32":
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-7)
+    else:
+        assert_half_close(got, want, ulps=1.0, frac=0.02, what="softmax")
+    assert np.all(got[0, :, 0, :] == 0)                      # fully masked row -> zeros (maximum clamped at 0)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("S,holes,weird", [(5, False, False), (32, False, False), (64, False, False),
+                                           (64, True, True), (100, True, False), (128, False, True), (21, True, True)])
+def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
+    print("attention", dtype, S, holes, weird, flush=True)
+    p = _attn_problem(S + 1, 5, S, 2, dtype, holes=holes, weird_mask=weird)
+    bi, wi, vwn = _idx_dev(p)
+    T, B, heads, d = p["T"], p["B"], p["heads"], p["d"]
+    H = heads * d
+    qp, kp, vp = o.add_qkv_bias_padding(p["q"], p["bq"], p["k"], p["bk"], p["v"], p["bv"], T, B, S, heads, d, p["bi"],
+                                        p["wi"], dtype)
+    want = o.attention(qp, kp, vp, p["attr"], T, p["bi"], p["wi"], dtype)
+    # layout 0: padded buffers
+    got0 = k.attention(dev(qp), dev(kp), dev(vp), 0, 0, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    # layout 1: packed [T,3H] rows with the bias already added
+    add = (lambda a, b: (a.astype(np.float32) + b.astype(np.float32)).astype(np.float32)) if dtype == "fp32" else o.hadd
+    packed = np.zeros((B * S, 3 * H), o._np_dtype(dtype))
+    packed[:T, :H] = add(p["q"], p["bq"]); packed[:T, H:2 * H] = add(p["k"], p["bk"]); packed[:T, 2 * H:] = add(p["v"], p["bv"])
+    pk = dev(packed)
+    got1 = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    assert np.array_equal(got0, got1)
+    assert np.all(got0[T:] == 0)
+    if dtype == "fp32":
+        np.testing.assert_allclose(got0[:T], want, rtol=1e-4, atol=2e-5)
+    else:
+        # fp32 accumulation vs the oracle's exact sums, three roundings to half on the way
+        np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
+
+
+# ---------------------------------------------------------------------------- GEMM ---
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("m,n,k_", [(1, 768, 768), (134, 768, 768), (257, 3072, 768), (300, 768, 3072),
+                                    (1000, 1024, 1024), (100, 200, 64), (70, 264, 128), (2000, 2304, 768)])
+def test_gemm(k, dtype, m, n, k_):
+    print("gemm", dtype, m, n, k_, flush=True)
+    rng = np.random.RandomState(m + n + k_)
+    a = o.rnd(rng.randn(m, k_), dtype)
+    b = o.rnd(0.05 * rng.randn(k_, n), dtype)
+    bias = o.rnd(rng.randn(n), dtype)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    got = k.gemm(dev(a), dev(b)).cpu().numpy()
+    scale = np.abs(exact).max()
+    if dtype == "fp32":
+        assert np.abs(got - exact).max() <= 1e-5 * scale
+    else:
+        assert np.all(np.abs(got.astype(np.float64) - exact) <= 0.51 * half_ulp(exact) + 1e-5 * scale)
+    # bias epilogue: element-type add on the rounded product
+    gotb = k.gemm(dev(a), dev(b), bias=dev(bias)).cpu().numpy()
+    if dtype == "fp32":
+        np.testing.assert_allclose(gotb, got + bias, rtol=1e-6, atol=1e-6)
+    else:
+        assert np.array_equal(gotb, o.hadd(got, bias))
+    # device-side row bound
+    if m > 10:
+        md = torch.tensor([m - 5], dtype=torch.int32, device="cuda")
+        got2 = k.gemm(dev(a), dev(b), m_dev=md).cpu().numpy()
+        assert np.array_equal(got2[:m - 5], got[:m - 5]) and np.all(got2[m - 5:] == 0)
