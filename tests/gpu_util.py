@@ -20,14 +20,14 @@ def half_ulp(x):
     return 2.0 ** (np.floor(np.log2(ax)) - 10)
 
 
-def assert_half_close(got, want, ulps=1.0, frac=0.02, what=""):
+def assert_half_close(got, want, ulps=1.0, frac=0.02, what="", atol=0.0):
     """got/want float16 arrays: every element within `ulps` half-ulps of want, and at most
     `frac` of the elements different at all."""
     g = np.asarray(got, dtype=np.float64)
     w = np.asarray(want, dtype=np.float64)
     assert g.shape == w.shape
     err = np.abs(g - w)
-    lim = ulps * half_ulp(w) * 1.001
+    lim = ulps * half_ulp(w) * 1.001 + atol
     bad = err > lim
     assert not bad.any(), "%s: %d elements beyond %.1f ulp, worst %g vs %g" % (
         what, bad.sum(), ulps, g[bad][0], w[bad][0])

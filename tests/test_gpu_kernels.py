@@ -142,7 +142,9 @@ def test_add_bias_act(k, dtype, m, n):
     if dtype == "fp32":
         np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
     else:
-        assert_half_close(got, want, ulps=1.0, frac=0.01, what="gelu")
+        # the CDF is rounded to half before the last multiply: a CDF one half-ulp off (exp2/rcp vs exact
+        # tanh) moves the product by up to 2 ulps, or by |x| * 2^-24 where the CDF is a half denormal
+        assert_half_close(got, want, ulps=2.0, frac=0.01, what="gelu", atol=1e-6)
     # rows bounded on the device: rows >= *m_dev stay untouched
     if m > 3:
         keep = torch.tensor([m - 2], dtype=torch.int32, device="cuda")
