@@ -223,6 +223,8 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
     return fail(h, ET_UNSUPPORTED, "attention kernel supports size_per_head == 64 and seq_len <= 128");
   if (!et::gemm_supported(dt, H, H, 3) || !et::gemm_supported(dt, F, H, 1) || !et::gemm_supported(dt, H, F, 1))
     return fail(h, ET_UNSUPPORTED, "hidden size not supported by the GEMM kernels");
+  if ((uint64_t)B * S * F * et::elem_size(dt) > 0xffffffffull)
+    return fail(h, ET_UNSUPPORTED, "activation matrix larger than 4 GB");
   if (!et::bias_gelu_supported(dt, F) || !et::bias_residual_layernorm_supported(dt, H))
     return fail(h, ET_UNSUPPORTED, "hidden size not supported by the row kernels");
   if (valid_word_num_hint == 0) return ET_OK;
@@ -455,6 +457,8 @@ et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, voi
   if (!et::gemm_supported(to_dt(dtype), n, k, 1))
     return fail(h, ET_UNSUPPORTED, dtype == ET_FP16 ? "fp16 GEMM needs k % 64 == 0 and n % 8 == 0"
                                                      : "fp32 GEMM needs k % 16 == 0 and n % 4 == 0");
+  if ((uint64_t)m * k * et::elem_size(to_dt(dtype)) > 0xffffffffull)
+    return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
   if (m == 0) return ET_OK;
   et::GemmGroups g;
   g.groups = 1;

@@ -6,10 +6,10 @@
 //
 // fp16: v_mfma_f32_16x16x32_f16.  B is n-contiguous in memory while the MFMA wants 8 consecutive k
 // per lane, so each lane reads an 8(k) x 8(n) block of B from LDS with eight 128-bit reads and
-// transposes it in registers; the eight resulting operands feed eight MFMAs whose column sets are
-// {8*l + j : l = 0..15}.  A lane therefore ends up owning 8 consecutive output columns per row and
-// stores C with 128-bit writes.  The k order inside a step is whatever the loads define; A and B use
-// the same one.
+// transposes it in registers (v_perm_b32); the eight resulting operands feed eight MFMAs whose column
+// sets are {8*l + j : l = 0..15}.  A lane therefore ends up owning 8 consecutive output columns per
+// row and stores C with 128-bit writes.  The k order inside a step is whatever the loads define; A and
+// B use the same one.
 // fp32: v_mfma_f32_32x32x2_f32, one element per lane per step.
 //
 // The M dimension (valid tokens) may live on the device: tiles beyond *rows_dev exit, the last tile
@@ -41,33 +41,66 @@ constexpr int kXcds = 8;
 __device__ __forceinline__ int remap_tile(int pid, int per_xcd) { return (pid % kXcds) * per_xcd + pid / kXcds; }
 
 // ------------------------------------------------------------------------------------------
-// fp16
+// fp16: (32*MI) x 256 tile, 4 wavefronts (2x2), k-step 32 = one v_mfma_f32_16x16x32_f16 depth.
+//
+// Global -> LDS goes through global_load_lds_dwordx4 (no register staging): one instruction moves
+// 64 lanes x 16 bytes into 1 KB of contiguous LDS, the lane chooses which 16-byte chunk of the tile it
+// fetches.  A rows are 64 bytes (4 chunks) per k-step; the chunk position inside a row is XOR-swizzled
+// with bits 1-2 of the row so that the MFMA operand reads (16 rows x one chunk per 16 lanes) spread
+// over the banks.  B keeps its natural [k][n] order.  A ring of kStages k-steps lives in LDS; the DMA
+// runs kStages-1 k-steps ahead of the MFMAs and is tracked with explicit vmcnt waits, the only
+// synchronisation per k-step is one s_barrier.  Operands of k-step t+1 are read from LDS and
+// transposed while the 8*MI MFMAs of k-step t issue.
 // ------------------------------------------------------------------------------------------
 constexpr int kHThreads = 256;
-constexpr int kHBK = 64;                  // k per LDS stage (two MFMA steps of 32)
-constexpr int kHAStride = kHBK + 8;       // halves; 144-byte rows: 16-byte reads of 8 consecutive rows hit distinct banks
+constexpr int kHBK = 32;
+constexpr int kHBN = 256;
+constexpr int kStages = 4;
 
-template <int MI, int WAVES_M, int WAVES_N>
+template <int MI>
 struct HTile {
-  static constexpr int BM = WAVES_M * 16 * MI;
-  static constexpr int BN = WAVES_N * 128;
-  static constexpr int A_CHUNKS = BM * (kHBK / 8) / kHThreads;    // 16-byte chunks per thread per stage
-  static constexpr int B_CHUNKS = kHBK * (BN / 8) / kHThreads;
-  static constexpr size_t A_BYTES = (size_t)BM * kHAStride * 2;
-  static constexpr size_t B_BYTES = (size_t)kHBK * BN * 2;
-  static constexpr size_t STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr size_t SMEM_BYTES = 2 * STAGE_BYTES;
-  static_assert(WAVES_M * WAVES_N * kWave == kHThreads, "4 wavefronts");
+  static constexpr int BM = 32 * MI;
+  static constexpr int A_BYTES = BM * kHBK * 2;
+  static constexpr int B_BYTES = kHBK * kHBN * 2;              // 16 KB
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int SMEM_BYTES = kStages * STAGE_BYTES;
+  static constexpr int A_DMA = A_BYTES / 1024 / 4;             // DMA instructions per wavefront per stage
+  static constexpr int B_DMA = B_BYTES / 1024 / 4;
+  static constexpr int DMA = A_DMA + B_DMA;
 };
 
-__device__ __forceinline__ uint32_t pack_lo(uint32_t x, uint32_t y) { return (x & 0xffffu) | (y << 16); }
-__device__ __forceinline__ uint32_t pack_hi(uint32_t x, uint32_t y) { return (x >> 16) | (y & 0xffff0000u); }
+#define ET_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-template <int MI, int WAVES_M, int WAVES_N>
+// gfx9 s_waitcnt immediate: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+template <int VM>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | (15 << 8) | ((VM >> 4) << 14));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14)); }
+// Barrier without the fence __syncthreads() carries: the fence would wait for every outstanding DMA.
+__device__ __forceinline__ void barrier_only() { asm volatile("s_barrier" ::: "memory"); }
+
+__device__ __forceinline__ int a_swizzle(int row) { return (row >> 1) & 3; }
+
+__device__ __forceinline__ void transpose8x8(const uint4v (&raw)[8], half8 (&bop)[8]) {
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) {       // dword jj of a raw k-row holds columns 2jj, 2jj+1
+    uint4v lo, hi;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      lo[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x05040100u);   // low halves
+      hi[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x07060302u);   // high halves
+    }
+    bop[2 * jj] = __builtin_bit_cast(half8, lo);
+    bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
+  }
+}
+
+template <int MI>
 __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
-  using Tile = HTile<MI, WAVES_M, WAVES_N>;
-  constexpr int BM = Tile::BM, BN = Tile::BN;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  using Tile = HTile<MI>;
+  constexpr int BM = Tile::BM, BN = kHBN;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tile = remap_tile(blockIdx.x, args.per_xcd);
   const int tiles_n_all = args.tiles_n * args.groups;
@@ -82,45 +115,47 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
   const int n0 = tn * BN;
   const int N = args.n, K = args.k;
 
-  const _Float16* __restrict__ A = (const _Float16*)args.A[grp];
-  const _Float16* __restrict__ B = (const _Float16*)args.B[grp];
-
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int wm = wave >> 1, wn = wave & 1;
   const int l16 = lane & 15, g = lane >> 4;
 
-  // global -> register staging
-  u32x4 ra[Tile::A_CHUNKS], rb[Tile::B_CHUNKS];
-  const int a_kc = tid & 7, a_row = tid >> 3;                 // + u*32
-  const int b_nc = tid % (BN / 8), b_krow = tid / (BN / 8);   // + u*(256/(BN/8))
-  constexpr int B_ROWS_PER_PASS = kHThreads / (BN / 8);
-  const bool b_col_ok = n0 + b_nc * 8 < N;
+  // Per-lane global byte offsets of the chunks this lane moves every stage.  Rows beyond the valid
+  // tokens and columns beyond N are clamped to valid addresses; what they load is never stored.
+  uint32_t a_off[Tile::A_DMA], b_off[Tile::B_DMA];
+#pragma unroll
+  for (int j = 0; j < Tile::A_DMA; ++j) {
+    const int q = wave * Tile::A_DMA + j;              // 1 KB slot of the A stage: 16 rows x 4 chunks
+    const int row = q * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ a_swizzle(row);
+    const int grow = min(m0 + row, rows - 1);
+    a_off[j] = ((uint32_t)grow * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+  }
+#pragma unroll
+  for (int j = 0; j < Tile::B_DMA; ++j) {
+    const int q = wave * Tile::B_DMA + j;              // 1 KB slot of the B stage: 2 k-rows x 32 chunks
+    const int kr = q * 2 + (lane >> 5);
+    const int col = min(n0 + (lane & 31) * 8, N - 8);
+    b_off[j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
+  }
+  const char* Ab = (const char*)args.A[grp];
+  const char* Bb = (const char*)args.B[grp];
+  const int nk = K / kHBK;
 
-  auto load_global = [&](int k0) {
+  auto issue = [&](int kt) {
+    unsigned char* st = smem + (kt % kStages) * Tile::STAGE_BYTES;
+    const int ktc = min(kt, nk - 1);       // past the end: re-load the last k-step (keeps the DMA count uniform)
+    const char* ab = Ab + (size_t)ktc * kHBK * 2;
+    const char* bb = Bb + (size_t)ktc * kHBK * N * 2;
 #pragma unroll
-    for (int u = 0; u < Tile::A_CHUNKS; ++u) {
-      const int row = m0 + a_row + u * 32;
-      ra[u] = u32x4{0u, 0u, 0u, 0u};
-      if (row < rows) ra[u] = *reinterpret_cast<const u32x4*>(A + (size_t)row * K + k0 + a_kc * 8);
-    }
+    for (int j = 0; j < Tile::A_DMA; ++j)
+      __builtin_amdgcn_global_load_lds((const void*)(ab + a_off[j]),
+                                       ET_LDS_PTR(st + (wave * Tile::A_DMA + j) * 1024), 16, 0, 0);
 #pragma unroll
-    for (int u = 0; u < Tile::B_CHUNKS; ++u) {
-      const int kr = k0 + b_krow + u * B_ROWS_PER_PASS;
-      rb[u] = u32x4{0u, 0u, 0u, 0u};
-      if (b_col_ok) rb[u] = *reinterpret_cast<const u32x4*>(B + (size_t)kr * N + n0 + b_nc * 8);
-    }
-  };
-  auto store_lds = [&](int stage) {
-    _Float16* As = reinterpret_cast<_Float16*>(smem + stage * Tile::STAGE_BYTES);
-    _Float16* Bs = reinterpret_cast<_Float16*>(smem + stage * Tile::STAGE_BYTES + Tile::A_BYTES);
-#pragma unroll
-    for (int u = 0; u < Tile::A_CHUNKS; ++u)
-      *reinterpret_cast<u32x4*>(As + (a_row + u * 32) * kHAStride + a_kc * 8) = ra[u];
-#pragma unroll
-    for (int u = 0; u < Tile::B_CHUNKS; ++u)
-      *reinterpret_cast<u32x4*>(Bs + (b_krow + u * B_ROWS_PER_PASS) * BN + b_nc * 8) = rb[u];
+    for (int j = 0; j < Tile::B_DMA; ++j)
+      __builtin_amdgcn_global_load_lds((const void*)(bb + b_off[j]),
+                                       ET_LDS_PTR(st + Tile::A_BYTES + (wave * Tile::B_DMA + j) * 1024), 16, 0, 0);
   };
 
   float4v acc[MI][8];
@@ -129,44 +164,61 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  const int nk = K / kHBK;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    if (kt + 1 < nk) load_global((kt + 1) * kHBK);
-    const _Float16* As = reinterpret_cast<const _Float16*>(smem + (kt & 1) * Tile::STAGE_BYTES);
-    const _Float16* Bs = reinterpret_cast<const _Float16*>(smem + (kt & 1) * Tile::STAGE_BYTES + Tile::A_BYTES);
+  // LDS read offsets in bytes: A row (wm*16*MI + i*16 + l16), chunk g (swizzled); B k-row g*8+kk, 8 columns
+  const int a_rd = ((wm * 16 * MI + l16) * 4 + (g ^ a_swizzle(l16))) * 16;
+  const int b_rd = ((g * 8) * BN + wn * 128 + l16 * 8) * 2;
+
 #pragma unroll
-    for (int ks = 0; ks < kHBK / 32; ++ks) {
-      // B: 8(k) x 8(n) block per lane, transposed in registers into 8 operands
-      uint4v raw[8];
+  for (int q = 0; q < kStages; ++q) issue(q);
+  wait_vmcnt<Tile::DMA * (kStages - 1)>();
+  barrier_only();
+  half8 a_cur[MI], bop_cur[8];
+  {
+    uint4v raw[8];
 #pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-        raw[kk] = *reinterpret_cast<const uint4v*>(Bs + (ks * 32 + g * 8 + kk) * BN + wn * 128 + l16 * 8);
-      half8 bop[8];
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint4v*>(smem + Tile::A_BYTES + b_rd + kk * BN * 2);
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {        // dword jj of a raw row holds columns 2jj, 2jj+1
-        uint4v lo, hi;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          lo[p] = pack_lo(raw[2 * p][jj], raw[2 * p + 1][jj]);
-          hi[p] = pack_hi(raw[2 * p][jj], raw[2 * p + 1][jj]);
-        }
-        bop[2 * jj] = __builtin_bit_cast(half8, lo);
-        bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
-      }
-#pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        const half8 a =
-            *reinterpret_cast<const half8*>(As + (wm * 16 * MI + i * 16 + l16) * kHAStride + ks * 32 + g * 8);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bop[j], acc[i][j], 0, 0, 0);
-      }
-    }
-    if (kt + 1 < nk) store_lds((kt + 1) & 1);
-    __syncthreads();
+    for (int i = 0; i < MI; ++i) a_cur[i] = *reinterpret_cast<const half8*>(smem + a_rd + i * 16 * 64);
+    transpose8x8(raw, bop_cur);
   }
+
+  for (int kt = 0; kt < nk; ++kt) {
+    wait_vmcnt<Tile::DMA * (kStages - 2)>();   // k-step kt+1 has landed; kt+2 and kt+3 may still be in flight
+    wait_lgkmcnt0();                           // this wavefront's reads of k-step kt's buffer are complete
+    barrier_only();
+    issue(kt + kStages);                       // into the buffer of k-step kt, free now for every wavefront
+    __builtin_amdgcn_sched_barrier(0);
+    const unsigned char* st = smem + ((kt + 1) % kStages) * Tile::STAGE_BYTES;
+    uint4v raw[8];
+    half8 a_n[MI], bop_n[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint4v*>(st + Tile::A_BYTES + b_rd + kk * BN * 2);
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a_n[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[i], bop_cur[j], acc[i][j], 0, 0, 0);
+    transpose8x8(raw, bop_n);
+    // issue order: LDS reads spread over the first half of the MFMAs, the transposes over the second half
+#pragma unroll
+    for (int r = 0; r < 8 + MI; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 LDS read
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
+    }
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);   // 1 VALU (transpose)
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a_cur[i] = a_n[i];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bop_cur[j] = bop_n[j];
+  }
+  wait_vmcnt<0>();        // no DMA may still target this workgroup's LDS when it ends
 
   // epilogue: lane owns rows g*4+r of every 16-row sub-tile and 8 consecutive columns
   const int col = n0 + wn * 128 + l16 * 8;
@@ -308,10 +360,10 @@ __global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
   }
 }
 
-template <int MI, int WAVES_M, int WAVES_N>
+template <int MI>
 void launch_f16(GemmArgs a, hipStream_t stream) {
-  using Tile = HTile<MI, WAVES_M, WAVES_N>;
-  auto kern = gemm_f16_kernel<MI, WAVES_M, WAVES_N>;
+  using Tile = HTile<MI>;
+  auto kern = gemm_f16_kernel<MI>;
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -319,7 +371,7 @@ void launch_f16(GemmArgs a, hipStream_t stream) {
     attr_set = true;
   }
   a.tiles_m = (a.m_bound + Tile::BM - 1) / Tile::BM;
-  a.tiles_n = (a.n + Tile::BN - 1) / Tile::BN;
+  a.tiles_n = (a.n + kHBN - 1) / kHBN;
   const int total = a.tiles_m * a.tiles_n * a.groups;
   a.per_xcd = (total + kXcds - 1) / kXcds;
   kern<<<a.per_xcd * kXcds, kHThreads, Tile::SMEM_BYTES, stream>>>(a);
@@ -329,7 +381,7 @@ void launch_f16(GemmArgs a, hipStream_t stream) {
 
 bool gemm_supported(DType t, int n, int k, int groups) {
   if (groups < 1 || groups > 3 || n <= 0 || k <= 0) return false;
-  if (t == DType::F16) return k % kHBK == 0 && n % 8 == 0;
+  if (t == DType::F16) return k % kHBK == 0 && n % 8 == 0 && n >= 8;
   return k % kFBK == 0 && n % 4 == 0;
 }
 
@@ -352,10 +404,10 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   if (t == DType::F16) {
     // few big tiles would leave most of the 256 CUs idle: fall back to 128-row tiles
     const long big = (long)((m_bound + 255) / 256) * ((n + 255) / 256) * g.groups;
-    if (big >= 512)
-      launch_f16<8, 2, 2>(a, stream);
+    if (big >= 256)
+      launch_f16<8>(a, stream);
     else
-      launch_f16<4, 2, 2>(a, stream);
+      launch_f16<4>(a, stream);
   } else {
     a.tiles_m = (m_bound + kFBM - 1) / kFBM;
     a.tiles_n = (n + kFBN - 1) / kFBN;
