@@ -43,9 +43,9 @@ __device__ __forceinline__ int remap_tile(int pid, int per_xcd) { return (pid % 
 // ------------------------------------------------------------------------------------------
 // fp16: (32*MI) x 256 tile, 4 wavefronts (2x2), k-step 32 = one v_mfma_f32_16x16x32_f16 depth.
 //
-// Global -> LDS goes through global_load_lds_dwordx4 (no register staging): one instruction moves
+// Global -> LDS goes through buffer_load_dwordx4 ... lds (no register staging): one instruction moves
 // 64 lanes x 16 bytes into 1 KB of contiguous LDS, the lane chooses which 16-byte chunk of the tile it
-// fetches.  A rows are 64 bytes (4 chunks) per k-step; the chunk position inside a row is XOR-swizzled
+// fetches (32-bit lane offset + scalar k offset against a buffer descriptor that bounds the rows).  A rows are 64 bytes (4 chunks) per k-step; the chunk position inside a row is XOR-swizzled
 // with bits 1-2 of the row so that the MFMA operand reads (16 rows x one chunk per 16 lanes) spread
 // over the banks.  B keeps its natural [k][n] order.  A ring of kStages k-steps lives in LDS; the DMA
 // runs kStages-1 k-steps ahead of the MFMAs and is tracked with explicit vmcnt waits, the only
@@ -98,6 +98,7 @@ __device__ __forceinline__ void transpose8x8(const uint4v (&raw)[8], half8 (&bop
 
 template <int MI>
 __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass only needs the stub
   using Tile = HTile<MI>;
   constexpr int BM = Tile::BM, BN = kHBN;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -117,20 +118,25 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // scalar: LDS targets of the DMA are SALU values
   const int wm = wave >> 1, wn = wave & 1;
   const int l16 = lane & 15, g = lane >> 4;
 
-  // Per-lane global byte offsets of the chunks this lane moves every stage.  Rows beyond the valid
-  // tokens and columns beyond N are clamped to valid addresses; what they load is never stored.
+  // Buffer descriptors bound the DMA: A rows at or beyond the valid-token count read as zero.
+  __amdgpu_buffer_rsrc_t rsrc_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(args.A[grp]), 0, (int)((uint32_t)rows * K * 2u), 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_b =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(args.B[grp]), 0, (int)((uint32_t)K * N * 2u), 0x00020000);
+
+  // Per-lane byte offsets of the chunks this lane moves every stage (the k offset is a scalar).
+  // Columns beyond N are clamped to a valid column; what they load is never stored.
   uint32_t a_off[Tile::A_DMA], b_off[Tile::B_DMA];
 #pragma unroll
   for (int j = 0; j < Tile::A_DMA; ++j) {
     const int q = wave * Tile::A_DMA + j;              // 1 KB slot of the A stage: 16 rows x 4 chunks
     const int row = q * 16 + (lane >> 2);
     const int c = (lane & 3) ^ a_swizzle(row);
-    const int grow = min(m0 + row, rows - 1);
-    a_off[j] = ((uint32_t)grow * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+    a_off[j] = ((uint32_t)(m0 + row) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
   }
 #pragma unroll
   for (int j = 0; j < Tile::B_DMA; ++j) {
@@ -139,23 +145,19 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
     const int col = min(n0 + (lane & 31) * 8, N - 8);
     b_off[j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
   }
-  const char* Ab = (const char*)args.A[grp];
-  const char* Bb = (const char*)args.B[grp];
   const int nk = K / kHBK;
 
   auto issue = [&](int kt) {
     unsigned char* st = smem + (kt % kStages) * Tile::STAGE_BYTES;
     const int ktc = min(kt, nk - 1);       // past the end: re-load the last k-step (keeps the DMA count uniform)
-    const char* ab = Ab + (size_t)ktc * kHBK * 2;
-    const char* bb = Bb + (size_t)ktc * kHBK * N * 2;
 #pragma unroll
     for (int j = 0; j < Tile::A_DMA; ++j)
-      __builtin_amdgcn_global_load_lds((const void*)(ab + a_off[j]),
-                                       ET_LDS_PTR(st + (wave * Tile::A_DMA + j) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, ET_LDS_PTR(st + (wave * Tile::A_DMA + j) * 1024), 16, a_off[j],
+                                               ktc * kHBK * 2, 0, 0);
 #pragma unroll
     for (int j = 0; j < Tile::B_DMA; ++j)
-      __builtin_amdgcn_global_load_lds((const void*)(bb + b_off[j]),
-                                       ET_LDS_PTR(st + Tile::A_BYTES + (wave * Tile::B_DMA + j) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, ET_LDS_PTR(st + Tile::A_BYTES + (wave * Tile::B_DMA + j) * 1024),
+                                               16, b_off[j], ktc * kHBK * N * 2, 0, 0);
   };
 
   float4v acc[MI][8];
@@ -237,10 +239,13 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) o[j] = f2h(acc[i][j][r]);
           if (has_bias) o = o + bias8;      // half add on the rounded product, as the reference's next kernel does
-          *reinterpret_cast<half8*>(C + (size_t)row * args.ldc) = o;
+          __builtin_nontemporal_store(o, reinterpret_cast<half8*>(C + (size_t)row * args.ldc));
         }
       }
   }
+#else
+  (void)args;
+#endif
 }
 
 // ------------------------------------------------------------------------------------------
