@@ -17,6 +17,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (FETCH_SIZE scaled by 2.0, the factor a
+# plain device copy of known size shows in the same run); cfg3 shapes.  (read + write) in bytes.
+MEASURED_TRAFFIC = {
+    ("cfg3", "gemm_ffn_up"): (369.1 + 236.7) * (1 << 20),
+    ("cfg3", "gemm_qkv"): (234.3 + 177.5) * (1 << 20),
+    ("cfg3", "bias_gelu"): (236.8 + 236.7) * (1 << 20),
+    ("cfg3", "bias_residual_layernorm"): (118.5 + 59.2) * (1 << 20),
+    ("cfg3", "attention"): (226.3 + 59.2) * (1 << 20),
+}
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"fp16": 2500.0, "fp32": 157.3}
 
@@ -120,6 +129,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--cpu-seqs", type=int, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every box here has one); --gpus %d is not supported" % a.gpus)
@@ -154,6 +165,12 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
     ms = s.elapsed_time(e) / a.steps
 
+    if a.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     kernels = {} if a.no_kernels else per_kernel(wl, T, w["mask"])
     roof = None
     if kernels:
@@ -163,7 +180,8 @@ def main():
         dom = max(share, key=share.get)
         kd = kernels[dom]
         roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved"], "peak": kd["peak"], "unit": kd["unit"],
-                "frac": kd["frac"], "traffic": None}
+                "frac": kd["frac"], "ms": kd["ms"],
+                "traffic": MEASURED_TRAFFIC.get((wl.name, dom))}
     cpu = None
     if not a.no_cpu:
         cpu = cpu_baseline(w, a.cpu_seqs or max(4, min(wl.B, 100 if wl.S <= 64 else 32)))
