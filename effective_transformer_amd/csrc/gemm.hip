@@ -14,6 +14,8 @@
 //
 // The M dimension (valid tokens) may live on the device: tiles beyond *rows_dev exit, the last tile
 // is predicated.  Up to three column groups (Q/K/V) share one launch.
+#include <algorithm>
+
 #include "et_device.hpp"
 #include "kernels.hpp"
 
@@ -249,6 +251,221 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
 }
 
 // ------------------------------------------------------------------------------------------
+// fp16, large problems: persistent 256 x 256 tiles, 8 wavefronts (two per SIMD) in opposite phases.
+//
+// Wave tile 128 x 64 (32 MFMAs per k-step, 128 accumulator registers), so two wavefronts fit one SIMD.
+// Waves 0-3 and 4-7 alternate: while one group issues its 32 MFMAs (raised priority) the other does
+// its fetch half of the k-step -- its share of the DMA for the k-step three ahead, the LDS operand
+// reads of the current k-step and the 8x4 B transpose -- and a barrier swaps the roles.  The MFMA pipe
+// of a SIMD therefore always has one wave feeding it and no wave needs a second operand register set.
+//
+// A workgroup walks its tiles (XCD-banded order) with ONE continuous DMA stream: the last k-steps of a
+// tile already fetch the first k-steps of the next one.  At a tile boundary a wave confirms every DMA
+// it has issued (vmcnt 0), then issues its C stores and carries on; the vmcnt waits that follow count
+// loads only (loads complete in order among themselves), so stores still in flight can delay such a
+// wait but never let it pass early.
+// ------------------------------------------------------------------------------------------
+constexpr int kPThreads = 512;
+constexpr int kPBM = 256, kPBN = 256;
+constexpr int kPStage = (kPBM * kHBK + kHBK * kPBN) * 2;      // 32 KB per k-step
+constexpr int kPSmem = kStages * kPStage;                     // 128 KB
+constexpr int kPABytes = kPBM * kHBK * 2;     // A part of a k-step slot, B follows
+
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+struct PTile {
+  int m0, n0, grp;
+};
+
+__global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs args) {
+#if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // 0..7, scalar
+  const int phase_group = wave >> 2;
+  const int wm = wave & 1, wn = (wave >> 1) & 3;                  // 128-row half, 64-column quarter of the tile
+  const int l16 = lane & 15, g = lane >> 4;
+  const int N = args.n, K = args.k;
+  const int nk = K / kHBK;
+
+  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
+  const int tiles_n_all = args.tiles_n * args.groups;
+  const int total = ((rows + kPBM - 1) / kPBM) * tiles_n_all;     // tiles that hold valid rows (a prefix in tile order)
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds;
+  const int G = gridDim.x;                                        // multiple of 8
+
+  // tile number `idx` of this workgroup's walk -> tile; every XCD owns a contiguous band of tiles
+  auto tile_id = [&](int idx) { return xcd * per_xcd + idx / kXcds; };
+  auto valid = [&](int idx) { return idx / kXcds < per_xcd && tile_id(idx) < total; };
+  auto locate = [&](int tile) {
+    PTile t;
+    const int tm = tile / tiles_n_all;
+    const int tn_all = tile - tm * tiles_n_all;
+    t.grp = tn_all / args.tiles_n;
+    t.m0 = tm * kPBM;
+    t.n0 = (tn_all - t.grp * args.tiles_n) * kPBN;
+    return t;
+  };
+
+  struct Src {
+    __amdgpu_buffer_rsrc_t a, b;
+    uint32_t off[4];        // 0,1: A chunks, 2,3: B chunks of this lane per k-step
+  };
+  auto make_src = [&](const PTile& t) {
+    Src s;
+    // descriptors bound the DMA: A rows at or beyond the valid-token count read as zero
+    s.a = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(args.A[t.grp]), 0, (int)((uint32_t)rows * K * 2u), 0x00020000);
+    s.b = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(args.B[t.grp]), 0, (int)((uint32_t)K * N * 2u), 0x00020000);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int q = wave * 2 + j;                      // 1 KB slot: A 16 rows x 4 chunks, B 2 k-rows x 32 chunks
+      const int row = q * 16 + (lane >> 2);
+      const int c = (lane & 3) ^ a_swizzle(row);
+      s.off[j] = ((uint32_t)(t.m0 + row) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+      const int kr = q * 2 + (lane >> 5);
+      const int pc = ((lane & 31) - 8 * ((kr >> 3) & 1)) & 31;   // B rows 8..15, 24..31 are rotated by 128 bytes in LDS
+      const int col = min(t.n0 + pc * 8, N - 8);                 // columns beyond N: a valid column, never stored
+      s.off[2 + j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
+    }
+    return s;
+  };
+  // this wave's share (4 of 32 instructions) of the DMA for k-step kt of a tile into ring slot `slot`
+  auto issue = [&](int slot, int kt, const Src& s) {
+    unsigned char* st = smem + slot * kPStage;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s.a, ET_LDS_PTR(st + (wave * 2 + j) * 1024), 16, s.off[j], kt * kHBK * 2,
+                                               0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, ET_LDS_PTR(st + kPABytes + (wave * 2 + j) * 1024), 16, s.off[2 + j],
+                                               kt * kHBK * N * 2, 0, 0);
+  };
+
+  // LDS operand addresses: A row (wm*128 + i*16 + l16), chunk g (swizzled); B k-row g*8+kk, 4 columns
+  const int a_rd = ((wm * 128 + l16) * 4 + (g ^ a_swizzle(l16))) * 16;
+  int b_rd[8];
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) {
+    const int row = g * 8 + kk;
+    b_rd[kk] = row * 512 + (((wn * 64 + l16 * 4) * 2 + 128 * ((row >> 3) & 1)) & 511);
+  }
+
+  int idx = blockIdx.x;
+  if (!valid(idx)) return;
+  PTile tile = locate(tile_id(idx));
+  Src cur = make_src(tile), nxt = cur;
+
+  float4v acc[8][4];
+  half8 a[8], bop[4];
+  int u = 0;                                   // k-steps done by this workgroup: ring slot of k-step = u & 3
+
+  auto fetch_phase = [&](int kt_issue, const Src& s, bool check) {
+    issue((u + 3) & 3, kt_issue, s);
+    const unsigned char* st = smem + (u & 3) * kPStage;
+    uint2v raw[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint2v*>(st + kPABytes + b_rd[kk]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {           // 8(k) x 4(n) block -> 4 operands
+      uint4v lo, hi;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        lo[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x05040100u);
+        hi[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x07060302u);
+      }
+      bop[2 * jj] = __builtin_bit_cast(half8, lo);
+      bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
+    }
+    if (check) wait_vmcnt<8>();                // this wave's share of k-step u+1 has landed (u+2, u+3 may fly)
+    wait_lgkmcnt0();
+  };
+  auto mfma_phase = [&](bool first) {
+    __builtin_amdgcn_s_setprio(1);
+    if (first) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], bop[j], float4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], bop[j], acc[i][j], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_setprio(0);
+  };
+
+  // k-steps beyond the tile (K < 96) re-load the last one; the data is never used
+  issue(0, 0, cur);
+  issue(1, min(1, nk - 1), cur);
+  issue(2, min(2, nk - 1), cur);
+  wait_vmcnt<8>();
+  barrier_only();
+  if (phase_group == 1) barrier_only();        // the second group runs one phase behind the first
+  bool first_tile = true;
+  while (true) {
+    const int nidx = idx + G;
+    const bool has_next = valid(nidx);
+    PTile ntile = tile;
+    if (has_next) {
+      ntile = locate(tile_id(nidx));
+      nxt = make_src(ntile);
+    } else {
+      nxt = cur;                               // re-loads of this tile keep the DMA count per k-step uniform
+    }
+    for (int t = 0; t < nk; ++t) {
+      // right after a tile boundary the first two k-steps were confirmed before the C stores went out
+      const bool check = first_tile || t >= 2;
+      if (t + 3 < nk) fetch_phase(t + 3, cur, check);
+      else fetch_phase(min(t + 3 - nk, nk - 1), nxt, check);
+      barrier_only();
+      mfma_phase(t == 0);
+      barrier_only();
+      ++u;
+    }
+    wait_vmcnt<0>();
+    {
+      const int col = tile.n0 + wn * 64 + l16 * 4;
+      if (col < N) {
+        _Float16* C = (_Float16*)args.C + (size_t)tile.grp * N + col;
+        half4 bias4;
+        const bool has_bias = args.bias[tile.grp] != nullptr;
+        if (has_bias) bias4 = *reinterpret_cast<const half4*>((const _Float16*)args.bias[tile.grp] + col);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = tile.m0 + wm * 128 + i * 16 + g * 4 + r;
+            if (row < rows) {
+              half4 o;
+#pragma unroll
+              for (int j = 0; j < 4; ++j) o[j] = f2h(acc[i][j][r]);
+              if (has_bias) o = o + bias4;     // half add on the rounded product, as the reference's next kernel does
+              __builtin_nontemporal_store(o, reinterpret_cast<half4*>(C + (size_t)row * args.ldc));
+            }
+          }
+      }
+    }
+    if (!has_next) break;
+    idx = nidx;
+    tile = ntile;
+    cur = nxt;
+    first_tile = false;
+  }
+  if (phase_group == 0) barrier_only();        // matches the extra barrier the second group started with
+  wait_vmcnt<0>();                             // no DMA may still target this workgroup's LDS when it ends
+#else
+  (void)args;
+#endif
+}
+
+// ------------------------------------------------------------------------------------------
 // fp32: 128x128x16 tile, 4 wavefronts (2x2) of 64x64, v_mfma_f32_32x32x2_f32
 // ------------------------------------------------------------------------------------------
 constexpr int kFThreads = 256;
@@ -382,6 +599,33 @@ void launch_f16(GemmArgs a, hipStream_t stream) {
   kern<<<a.per_xcd * kXcds, kHThreads, Tile::SMEM_BYTES, stream>>>(a);
 }
 
+int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+void launch_f16_persistent(GemmArgs a, hipStream_t stream) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_persistent_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kPSmem);
+    attr_set = true;
+  }
+  a.tiles_m = (a.m_bound + kPBM - 1) / kPBM;
+  a.tiles_n = (a.n + kPBN - 1) / kPBN;
+  const int total = a.tiles_m * a.tiles_n * a.groups;
+  int grid = std::min(device_cu_count(), total);
+  grid = (grid + kXcds - 1) / kXcds * kXcds;
+  a.per_xcd = 0;     // derived on the device from the valid row count
+  gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
+}
+
 }  // namespace
 
 bool gemm_supported(DType t, int n, int k, int groups) {
@@ -409,10 +653,10 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   if (t == DType::F16) {
     // few big tiles would leave most of the 256 CUs idle: fall back to 128-row tiles
     const long big = (long)((m_bound + 255) / 256) * ((n + 255) / 256) * g.groups;
-    if (big >= 256)
-      launch_f16<8>(a, stream);
+    if (big >= 128 && k >= 4 * kHBK)
+      launch_f16_persistent(a, stream);      // one workgroup per CU walks the tiles
     else
-      launch_f16<4>(a, stream);
+      launch_f16<4>(a, stream);              // few tiles: 128-row tiles spread over more CUs
   } else {
     a.tiles_m = (m_bound + kFBM - 1) / kFBM;
     a.tiles_n = (n + kFBN - 1) / kFBN;
