@@ -21,10 +21,12 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 template <typename T> struct Chunk16;
 template <> struct Chunk16<float> {
+  typedef float4v vec;
   float4v v;
   static constexpr int kElems = 4;
 };
 template <> struct Chunk16<_Float16> {
+  typedef half8 vec;
   half8 v;
   static constexpr int kElems = 8;
 };
@@ -145,10 +147,12 @@ __global__ __launch_bounds__(256) void transpose_rm_padding_kernel(
 // ------------------------------------------------------------------------------------------
 // fused attention, size_per_head = 64, seq_len <= 128.
 //
-// One workgroup (4 wavefronts) per (sequence, head).  The sequence's K rows and the transpose of
-// its V rows are staged in LDS at their padded positions (zero where no token exists, so that a
-// mask that attends to a padded key sees the zero score / zero value the reference's padded
-// buffers hold); Q rows are staged beside them.  Each wavefront takes 16-query tiles:
+// One workgroup (4 wavefronts) per (sequence, group of up to 4 heads).  What does not depend on the
+// head is done once: token positions, the zero fill of key/value slots without a token (so that a
+// mask that attends to a padded key sees the zero score / zero value the reference's padded buffers
+// hold) and the mask rows of each wavefront's queries, which stay in registers.  Per head the K rows
+// and the transpose of the V rows are staged in LDS at their padded positions, Q rows beside them,
+// while the next head's rows are already in flight into registers.  Each wavefront takes 16-query tiles:
 //   S^T = K Q^T   on v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x4_f32 -> a lane owns one query
 //                 column and 4 keys of every 16-key tile,
 //   softmax       over the lane's values + 2 cross-lane steps (lanes l, l^16, l^32, l^48 share a query),
@@ -191,11 +195,13 @@ __device__ __forceinline__ float xor_lanes_16_32_sum(float v) {
   return v;
 }
 
-template <typename T, int NKT>
+// CPT = 16-byte chunks of one matrix a thread moves per head (ceil(seq rows * chunks per row / 256)).
+// PF: keep the next head's Q/K/V chunks in registers while the current head is computed.
+template <typename T, int NKT, int CPT, bool PF>
 __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
-    const int32_t* __restrict__ word_idx, int seq_len, int heads, float scaler) {
+    const int32_t* __restrict__ word_idx, int seq_len, int heads, int heads_per_wg, float scaler) {
   using Cfg = AttnCfg<T>;
   using Sm = AttnSmem<T, NKT>;
   using C = Chunk16<T>;
@@ -203,6 +209,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   constexpr int kVS = Sm::kVtStride;
   constexpr int kSp = Sm::kSp;
   constexpr int kCpr = kD / C::kElems;       // 16-byte chunks per head row
+  constexpr int QPW = NKT > 4 ? NKT / 4 : 1; // query tiles per wavefront
+  typedef T mask4 __attribute__((ext_vector_type(4)));
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* Qs = reinterpret_cast<T*>(smem_raw);
@@ -210,219 +218,276 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   T* Vt = reinterpret_cast<T*>(smem_raw + 2 * Sm::kQBytes);
   int* tok_of_pos = reinterpret_cast<int*>(smem_raw + 2 * Sm::kQBytes + Sm::kVtBytes);
 
-  const int head = blockIdx.x;
   const int b = blockIdx.y;
+  const int h_begin = blockIdx.x * heads_per_wg;
+  const int h_end = min(h_begin + heads_per_wg, heads);
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
   const int len = t1 - t0;
   if (len <= 0) return;
   const int H = heads * kD;
-  // positions are ascending inside a sequence: the last token bounds the occupied tiles
-  const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
-  const int n_tiles = last_pos / 16 + 1;    // 16-row tiles that hold at least one token (queries and keys)
-
-  // ---- stage: zero the key/value tiles in use, then scatter the sequence's rows --------------
-  for (int i = threadIdx.x; i < kSp; i += kAttnThreads) tok_of_pos[i] = -1;
-  {
-    const int rows = n_tiles * 16;
-    uint32_t* kz = reinterpret_cast<uint32_t*>(Ks);
-    const int kwords = rows * kQS * (int)sizeof(T) / 4;
-    for (int i = threadIdx.x; i < kwords; i += kAttnThreads) kz[i] = 0u;
-    uint32_t* vz = reinterpret_cast<uint32_t*>(Vt);
-    const int vwords = kD * kVS * (int)sizeof(T) / 4;
-    for (int i = threadIdx.x; i < vwords; i += kAttnThreads) vz[i] = 0u;
-  }
-  __syncthreads();
-  for (int i = threadIdx.x; i < len * kCpr; i += kAttnThreads) {
-    const int tt = i / kCpr;
-    const int c = i - tt * kCpr;
-    const int t = t0 + tt;
-    const int pos = word_idx[t];
-    if (pos < 0 || pos >= seq_len) continue;
-    size_t off;
-    if (layout == 1) {
-      off = (size_t)t * packed_ld + head * kD + c * C::kElems;
-    } else {
-      off = (((size_t)b * heads + head) * seq_len + pos) * kD + c * C::kElems;
-    }
-    const C qv = *reinterpret_cast<const C*>(q_src + off);
-    const C kv = *reinterpret_cast<const C*>(k_src + off);
-    const C vv = *reinterpret_cast<const C*>(v_src + off);
-    *reinterpret_cast<C*>(Qs + pos * kQS + c * C::kElems) = qv;
-    *reinterpret_cast<C*>(Ks + pos * kQS + c * C::kElems) = kv;
-#pragma unroll
-    for (int j = 0; j < C::kElems; ++j) Vt[(c * C::kElems + j) * kVS + pos] = vv.v[j];
-    if (c == 0) tok_of_pos[pos] = t;
-  }
-  __syncthreads();
-
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int l16 = lane & 15;
   const int g = lane >> 4;
 
-  for (int qt = wave; qt < n_tiles; qt += kAttnWaves) {
-    const int q = qt * 16 + l16;            // this lane's query position
-    float s[NKT][4];
-    // ---- S^T = K Q^T -------------------------------------------------------------------
-    if constexpr (sizeof(T) == 2) {
-      half8 bq[2];
+  // ---- everything that does not depend on the head: issued up front, all loads in flight together ----
+  // positions are ascending inside a sequence: the last token bounds the occupied 16-row tiles
+  const int last_pos_raw = word_idx[t1 - 1];
+  int my_t[CPT], my_pos[CPT], my_c[CPT];
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) bq[ks] = *reinterpret_cast<const half8*>(Qs + q * kQS + ks * 32 + g * 8);
+  for (int k = 0; k < CPT; ++k) {
+    const int i = threadIdx.x + k * kAttnThreads;
+    const int tt = i / kCpr;
+    my_c[k] = i - tt * kCpr;
+    my_t[k] = tt < len ? t0 + tt : -1;
+    my_pos[k] = tt < len ? word_idx[t0 + tt] : -1;
+  }
+  // the mask rows of this wavefront's queries stay in registers for all heads
+  mask4 mreg[QPW][NKT];
+  const bool vec_mask = (seq_len & 3) == 0;
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) {
-        float4v acc = {0.f, 0.f, 0.f, 0.f};
-        if (kt < n_tiles) {
-#pragma unroll
-          for (int ks = 0; ks < 2; ++ks) {
-            const half8 a = *reinterpret_cast<const half8*>(Ks + (kt * 16 + l16) * kQS + ks * 32 + g * 8);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bq[ks], acc, 0, 0, 0);
-          }
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s[kt][r] = h2f(f2h(acc[r]));   // the score is stored in half
-      }
-    } else {
-      float bq[16];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float4v v4 = *reinterpret_cast<const float4v*>(Qs + q * kQS + g * 16 + i * 4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) bq[i * 4 + j] = v4[j];
-      }
-#pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) {
-        float4v acc = {0.f, 0.f, 0.f, 0.f};
-        if (kt < n_tiles) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kt * 16 + l16) * kQS + g * 16 + i * 4);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bq[i * 4 + j], acc, 0, 0, 0);
-          }
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s[kt][r] = acc[r];
-      }
-    }
-    // ---- masked softmax over the keys of query q ------------------------------------------
-    const bool q_ok = q < seq_len;
-    const T* mrow = attr_mask + ((size_t)b * seq_len + (q_ok ? q : 0)) * seq_len;
-    float mx = 0.f;                          // clamp of the maximum at 0
-    const bool vec_mask = (seq_len & 3) == 0;
+  for (int qi = 0; qi < QPW; ++qi) {
+    const int q = (wave + qi * kAttnWaves) * 16 + l16;
+    const T* mrow = attr_mask + ((size_t)b * seq_len + min(q, seq_len - 1)) * seq_len;
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) {
       const int key0 = kt * 16 + g * 4;
-      float mval[4] = {0.f, 0.f, 0.f, 0.f};
+      mask4 m4 = {(T)0, (T)0, (T)0, (T)0};
       if (vec_mask) {
-        if (key0 < seq_len) {
-          typedef T mask4 __attribute__((ext_vector_type(4)));
-          const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + key0);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) mval[r] = (float)m4[r];
-        }
+        if (key0 < seq_len) m4 = *reinterpret_cast<const mask4*>(mrow + key0);
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (key0 + r < seq_len) mval[r] = (float)mrow[key0 + r];
+          if (key0 + r < seq_len) m4[r] = mrow[key0 + r];
       }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        // keys beyond seq_len do not exist
-        const float tv = key0 + r < seq_len ? s[kt][r] * scaler + (1.0f - mval[r]) * -10000.0f : -INFINITY;
-        s[kt][r] = tv;
-        mx = fmaxf(mx, tv);
-      }
+      mreg[qi][kt] = m4;
     }
-    mx = xor_lanes_16_32_max(mx);
-    float sum = 0.f;
+  }
+  using V16 = typename C::vec;
+  V16 rq[CPT], rk[CPT], rv[CPT];
+  // 16-byte chunk k of this thread for `head`: element offset into the source matrices
+#define ET_ATTN_LOAD_HEAD(head_)                                                                            \
+  _Pragma("unroll") for (int k = 0; k < CPT; ++k) {                                                         \
+    if (my_t[k] >= 0 && my_pos[k] >= 0 && my_pos[k] < seq_len) {                                            \
+      const size_t off = layout == 1                                                                        \
+                             ? (size_t)my_t[k] * packed_ld + (head_) * kD + my_c[k] * C::kElems             \
+                             : (((size_t)b * heads + (head_)) * seq_len + my_pos[k]) * kD + my_c[k] * C::kElems; \
+      rq[k] = *reinterpret_cast<const V16*>(q_src + off);                                                   \
+      rk[k] = *reinterpret_cast<const V16*>(k_src + off);                                                   \
+      rv[k] = *reinterpret_cast<const V16*>(v_src + off);                                                   \
+    }                                                                                                       \
+  }
+  if (PF) { ET_ATTN_LOAD_HEAD(h_begin) }
+
+  const int last_pos = min(max(last_pos_raw, 0), seq_len - 1);
+  const int n_tiles = last_pos / 16 + 1;    // 16-row tiles that hold at least one token (queries and keys)
+
+  // ---- position table, then zero the key / value slots that hold no token (once: heads only overwrite tokens) ----
+  for (int i = threadIdx.x; i < kSp; i += kAttnThreads) tok_of_pos[i] = -1;
+  __syncthreads();
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        s[kt][r] = __builtin_amdgcn_exp2f((s[kt][r] - mx) * kLog2e);
-        sum += s[kt][r];
-      }
-    sum = xor_lanes_16_32_sum(sum) + 1e-6f;
-    const float inv = 1.0f / sum;
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
-    // ---- O^T = V^T P^T --------------------------------------------------------------------
-    float4v o[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-      for (int ks = 0; ks < NKT / 2; ++ks) {
-        if (2 * ks < n_tiles) {
-          half8 p;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            p[r] = f2h(s[2 * ks][r]);
-            p[4 + r] = f2h(s[2 * ks + 1][r]);
-          }
-#pragma unroll
-          for (int dt = 0; dt < 4; ++dt) {
-            const T* vrow = Vt + (dt * 16 + l16) * kVS + ks * 32 + g * 4;
-            const half4 lo = *reinterpret_cast<const half4*>(vrow);
-            const half4 hi = *reinterpret_cast<const half4*>(vrow + 16);
-            half8 a;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              a[r] = lo[r];
-              a[4 + r] = hi[r];
-            }
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, p, o[dt], 0, 0, 0);
-          }
+  for (int k = 0; k < CPT; ++k)
+    if (my_t[k] >= 0 && my_c[k] == 0 && my_pos[k] >= 0 && my_pos[k] < seq_len) tok_of_pos[my_pos[k]] = my_t[k];
+  __syncthreads();
+  {
+    // the fp16 P.V contraction runs over pairs of key tiles, so an odd tile count drags one more tile of Vt in
+    const int rows = min(kSp, ((n_tiles + 1) / 2) * 32);
+    // K: row `pos` (kQS elements), Vt: column `pos` of every feature row
+    for (int i = threadIdx.x; i < rows * (kD / 2); i += kAttnThreads) {
+      const int pos = i / (kD / 2), w = i - pos * (kD / 2);
+      if (tok_of_pos[pos] < 0) {
+        if (sizeof(T) == 2) {
+          reinterpret_cast<uint32_t*>(Ks + pos * kQS)[w] = 0u;                // 2 halves
+          Vt[(2 * w) * kVS + pos] = (T)0;
+          Vt[(2 * w + 1) * kVS + pos] = (T)0;
+        } else {
+          Ks[pos * kQS + 2 * w] = (T)0; Ks[pos * kQS + 2 * w + 1] = (T)0;
+          Vt[(2 * w) * kVS + pos] = (T)0;
+          Vt[(2 * w + 1) * kVS + pos] = (T)0;
         }
       }
-    } else {
+    }
+  }
+
+  for (int head = h_begin; head < h_end; ++head) {
+    if (!PF) { ET_ATTN_LOAD_HEAD(head) }
+    if (head != h_begin) __syncthreads();      // every wavefront is done with the previous head's tiles
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+      const int pos = my_pos[k];
+      if (my_t[k] >= 0 && pos >= 0 && pos < seq_len) {
+        const int c = my_c[k];
+        *reinterpret_cast<V16*>(Qs + pos * kQS + c * C::kElems) = rq[k];
+        *reinterpret_cast<V16*>(Ks + pos * kQS + c * C::kElems) = rk[k];
+#pragma unroll
+        for (int j = 0; j < C::kElems; ++j) Vt[(c * C::kElems + j) * kVS + pos] = rv[k][j];
+      }
+    }
+    __syncthreads();
+    if (PF && head + 1 < h_end) { ET_ATTN_LOAD_HEAD(head + 1) }   // flies while this head is computed
+
+#pragma unroll
+    for (int qi = 0; qi < QPW; ++qi) {
+      const int qt = wave + qi * kAttnWaves;
+      if (qt >= n_tiles) break;               // wave-uniform
+      const int q = qt * 16 + l16;            // this lane's query position
+      float s[NKT][4];
+      // ---- S^T = K Q^T -------------------------------------------------------------------
+      if constexpr (sizeof(T) == 2) {
+        half8 bq[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) bq[ks] = *reinterpret_cast<const half8*>(Qs + q * kQS + ks * 32 + g * 8);
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt) {
+          float4v acc = {0.f, 0.f, 0.f, 0.f};
+          if (kt < n_tiles) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+              const half8 a = *reinterpret_cast<const half8*>(Ks + (kt * 16 + l16) * kQS + ks * 32 + g * 8);
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bq[ks], acc, 0, 0, 0);
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[kt][r] = h2f(f2h(acc[r]));   // the score is stored in half
+        }
+      } else {
+        float bq[16];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float4v v4 = *reinterpret_cast<const float4v*>(Qs + q * kQS + g * 16 + i * 4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) bq[i * 4 + j] = v4[j];
+        }
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt) {
+          float4v acc = {0.f, 0.f, 0.f, 0.f};
+          if (kt < n_tiles) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kt * 16 + l16) * kQS + g * 16 + i * 4);
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bq[i * 4 + j], acc, 0, 0, 0);
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[kt][r] = acc[r];
+        }
+      }
+      // ---- masked softmax over the keys of query q ------------------------------------------
+      float mx = 0.f;                          // clamp of the maximum at 0
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt) {
-        if (kt < n_tiles) {
+        const int key0 = kt * 16 + g * 4;
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt) {
-            const float4v a4 = *reinterpret_cast<const float4v*>(Vt + (dt * 16 + l16) * kVS + kt * 16 + g * 4);
+        for (int r = 0; r < 4; ++r) {
+          // keys beyond seq_len do not exist
+          const float tv = key0 + r < seq_len
+                               ? s[kt][r] * scaler + (1.0f - (float)mreg[qi][kt][r]) * -10000.0f
+                               : -INFINITY;
+          s[kt][r] = tv;
+          mx = fmaxf(mx, tv);
+        }
+      }
+      mx = xor_lanes_16_32_max(mx);
+      float sum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[kt][r], o[dt], 0, 0, 0);
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          s[kt][r] = __builtin_amdgcn_exp2f((s[kt][r] - mx) * kLog2e);
+          sum += s[kt][r];
+        }
+      sum = xor_lanes_16_32_sum(sum) + 1e-6f;
+      const float inv = 1.0f / sum;
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
+      // ---- O^T = V^T P^T --------------------------------------------------------------------
+      float4v o[4];
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+      if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int ks = 0; ks < NKT / 2; ++ks) {
+          if (2 * ks < n_tiles) {
+            half8 p;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              p[r] = f2h(s[2 * ks][r]);
+              p[4 + r] = f2h(s[2 * ks + 1][r]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+              const T* vrow = Vt + (dt * 16 + l16) * kVS + ks * 32 + g * 4;
+              const half4 lo = *reinterpret_cast<const half4*>(vrow);
+              const half4 hi = *reinterpret_cast<const half4*>(vrow + 16);
+              half8 a;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                a[r] = lo[r];
+                a[4 + r] = hi[r];
+              }
+              o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, p, o[dt], 0, 0, 0);
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt) {
+          if (kt < n_tiles) {
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+              const float4v a4 = *reinterpret_cast<const float4v*>(Vt + (dt * 16 + l16) * kVS + kt * 16 + g * 4);
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[kt][r], o[dt], 0, 0, 0);
+            }
           }
         }
       }
-    }
-    // ---- write the lane's 4x4 features of its query's packed row --------------------------
-    const int tq = q < kSp ? tok_of_pos[q] : -1;
-    if (tq >= 0) {
-      T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+      // ---- write the lane's 4x4 features of its query's packed row --------------------------
+      const int tq = tok_of_pos[q];
+      if (tq >= 0) {
+        T* orow = dst + (size_t)tq * H + head * kD + g * 4;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        typedef T out4 __attribute__((ext_vector_type(4)));
-        out4 v;
+        for (int dt = 0; dt < 4; ++dt) {
+          typedef T out4 __attribute__((ext_vector_type(4)));
+          out4 v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (T)o[dt][r];
-        *reinterpret_cast<out4*>(orow + dt * 16) = v;
+          for (int r = 0; r < 4; ++r) v[r] = (T)o[dt][r];
+          *reinterpret_cast<out4*>(orow + dt * 16) = v;
+        }
       }
     }
   }
 }
+
+#undef ET_ATTN_LOAD_HEAD
 
 template <typename T, int NKT>
 void attention_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                       void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                       float scaler, hipStream_t stream) {
   using Sm = AttnSmem<T, NKT>;
-  auto kern = attention_kernel<T, NKT>;
+  constexpr int kCpr = kD * (int)sizeof(T) / 16;
+  constexpr int CPT = (NKT * 16 * kCpr + kAttnThreads - 1) / kAttnThreads;
+  constexpr bool PF = CPT <= 4;                // more than 4 chunks x 3 matrices in flight would not fit the registers
+  auto kern = attention_kernel<T, NKT, CPT, PF>;
   static bool attr_set = false;
   if (!attr_set) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)Sm::kBytes);
     attr_set = true;
   }
-  dim3 grid(heads, batch);
+  // a workgroup serves up to 4 heads of one sequence: mask rows, positions and zero fill are shared by them
+  int hpw = 4;
+  while (hpw > 1 && (long)batch * ((heads + hpw - 1) / hpw) < 2048) hpw >>= 1;   // small batches: more workgroups
+  dim3 grid((heads + hpw - 1) / hpw, batch);
   kern<<<grid, kAttnThreads, Sm::kBytes, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
                                                    (const T*)attr_mask, (T*)dst, seq_start, word_idx, seq_len, heads,
-                                                   scaler);
+                                                   hpw, scaler);
 }
 
 template <typename T>

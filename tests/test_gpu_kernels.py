@@ -267,6 +267,26 @@ def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
         np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_fused_attention_many_sequences_head_groups(k, dtype):
+    """A batch large enough that one workgroup serves a group of 4 heads (shared mask registers, positions and
+    zero fill across heads, next head prefetched): holes in the mask, an attention mask unrelated to it."""
+    S, heads, B = 16, 12, 720
+    p = _attn_problem(99, B, S, heads, dtype, holes=True, weird_mask=True)
+    bi, wi, vwn = _idx_dev(p)
+    T, d = p["T"], p["d"]
+    H = heads * d
+    qp, kp, vp = o.add_qkv_bias_padding(p["q"], p["bq"], p["k"], p["bk"], p["v"], p["bv"], T, B, S, heads, d, p["bi"],
+                                        p["wi"], dtype)
+    want = o.attention(qp, kp, vp, p["attr"], T, p["bi"], p["wi"], dtype)
+    got0 = k.attention(dev(qp), dev(kp), dev(vp), 0, 0, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    assert np.all(got0[T:] == 0)
+    if dtype == "fp32":
+        np.testing.assert_allclose(got0[:T], want, rtol=1e-4, atol=2e-5)
+    else:
+        np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
+
+
 # ---------------------------------------------------------------------------- GEMM ---
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
