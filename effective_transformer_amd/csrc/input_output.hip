@@ -59,7 +59,26 @@ __global__ __launch_bounds__(kScanThreads) void scan_index_kernel(const int32_t*
   __shared__ int lds[kScanWaves];
   __shared__ int wave_tot[kScanWaves];
   int part = 0;
-  for (int i = threadIdx.x; i < (int)blockIdx.x; i += kScanThreads) part += sums[i];
+  if (sums) {
+    for (int i = threadIdx.x; i < (int)blockIdx.x; i += kScanThreads) part += sums[i];
+  } else {
+    // few tiles: add up everything in front of this tile straight from the input (it sits in L2), saving a launch
+    const int n4 = blockIdx.x * tile / 4;             // int4 words in front of this tile (tile is a multiple of 4)
+    const int4* in4 = reinterpret_cast<const int4*>(in);
+    constexpr int kU = 8;                             // independent loads in flight per thread
+    int i = threadIdx.x;
+    for (; i + (kU - 1) * kScanThreads < n4; i += kU * kScanThreads) {
+      int4 v[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) v[u] = in4[i + u * kScanThreads];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) part += v[u].x + v[u].y + v[u].z + v[u].w;
+    }
+    for (; i < n4; i += kScanThreads) {
+      const int4 v = in4[i];
+      part += v.x + v.y + v.z + v.w;
+    }
+  }
   int carry = block_sum_i32(part, lds);
 
   const int begin = blockIdx.x * tile;
@@ -128,22 +147,29 @@ __global__ __launch_bounds__(kMoveThreads) void compress_rows_kernel(
   T = min(T, n_pos);
   const uint32_t total = (uint32_t)T * cpr.d;
   const uint32_t base = blockIdx.x * (kMoveThreads * kMoveUnroll) + threadIdx.x;
-  u32x4 val[kMoveUnroll];
-  uint32_t dst[kMoveUnroll];
+  if (blockIdx.x * (kMoveThreads * kMoveUnroll) >= total) return;
+  // No predication at all: lanes past the end repeat the last chunk (load and store of identical data), so that
+  // all index loads, then all data loads, then all stores are issued back to back.
+  const uint32_t last = total - 1;
+  uint32_t row[kMoveUnroll], chunk[kMoveUnroll], idx[kMoveUnroll];
+  int bi[kMoveUnroll], wi[kMoveUnroll];
 #pragma unroll
   for (int u = 0; u < kMoveUnroll; ++u) {
-    const uint32_t i = base + u * kMoveThreads;
-    dst[u] = i;
-    if (i < total) {
-      const uint32_t t = div_by(i, cpr);
-      const uint32_t c = i - t * cpr.d;
-      const uint32_t src_row = (uint32_t)batch_idx[t] * (uint32_t)seq_len + (uint32_t)word_idx[t];
-      val[u] = from[(size_t)src_row * cpr.d + c];
-    }
+    const uint32_t i = min(base + u * kMoveThreads, last);
+    idx[u] = i;
+    row[u] = div_by(i, cpr);
+    chunk[u] = i - row[u] * cpr.d;
+    bi[u] = batch_idx[row[u]];
+    wi[u] = word_idx[row[u]];
+  }
+  u32x4 val[kMoveUnroll];
+#pragma unroll
+  for (int u = 0; u < kMoveUnroll; ++u) {
+    const uint32_t src_row = (uint32_t)bi[u] * (uint32_t)seq_len + (uint32_t)wi[u];
+    val[u] = from[(size_t)src_row * cpr.d + chunk[u]];
   }
 #pragma unroll
-  for (int u = 0; u < kMoveUnroll; ++u)
-    if (dst[u] < total) to[dst[u]] = val[u];
+  for (int u = 0; u < kMoveUnroll; ++u) to[idx[u]] = val[u];
 }
 
 constexpr int kRestorePos = 32;   // padded positions per workgroup
@@ -238,9 +264,12 @@ void launch_scan_index(const int32_t* in, int length, int32_t* prefix_out, int32
                        int32_t* valid_word_num, int seq_len, int32_t* scratch, hipStream_t stream) {
   const int tile = scan_tile_for(length);
   const int tiles = (length + tile - 1) / tile;
-  if (tiles > 1) scan_tile_sums_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, scratch);
-  scan_index_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, scratch, prefix_out, batch_idx, word_idx,
-                                                         valid_word_num, seq_len);
+  // up to 256 tiles every workgroup re-adds the elements in front of its tile itself (at most 1 MB of L2 reads);
+  // beyond that a first kernel leaves the tile totals in the scratch
+  const bool direct = tiles <= 128 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+  if (!direct) scan_tile_sums_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, scratch);
+  scan_index_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, direct ? nullptr : scratch, prefix_out,
+                                                         batch_idx, word_idx, valid_word_num, seq_len);
 }
 
 void launch_index_from_prefix(const int32_t* mask, const int32_t* prefix, int32_t* batch_idx, int32_t* word_idx,

@@ -65,15 +65,19 @@ __global__ __launch_bounds__(kGeluThreads) void bias_gelu_kernel(T* __restrict__
   const int r1 = min(r0 + kGeluRows, rows);
   for (int r = r0; r < r1; r += kGeluInFlight) {
     Chunk x[kGeluInFlight];
+    // no predication: rows past the end repeat the last row (same input, same result, same store), so the four
+    // loads are in flight together
+    Chunk* p[kGeluInFlight];
 #pragma unroll
-    for (int u = 0; u < kGeluInFlight; ++u)
-      if (r + u < r1) x[u] = base[(size_t)(r + u) * cpr];
+    for (int u = 0; u < kGeluInFlight; ++u) {
+      p[u] = base + (size_t)min(r + u, r1 - 1) * cpr;
+      x[u] = *p[u];
+    }
 #pragma unroll
-    for (int u = 0; u < kGeluInFlight; ++u)
-      if (r + u < r1) {
-        x[u].apply(b);
-        base[(size_t)(r + u) * cpr] = x[u];
-      }
+    for (int u = 0; u < kGeluInFlight; ++u) {
+      x[u].apply(b);
+      *p[u] = x[u];
+    }
   }
 }
 
