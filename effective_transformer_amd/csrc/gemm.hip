@@ -16,6 +16,8 @@
 // is predicated.  Up to three column groups (Q/K/V) share one launch.
 #include <algorithm>
 
+#include <type_traits>
+
 #include "et_device.hpp"
 #include "kernels.hpp"
 
@@ -431,25 +433,33 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
     }
     wait_vmcnt<0>();
     {
+      // C goes out through a buffer descriptor that ends at the last valid row: rows beyond it are dropped by
+      // the bounds check, and the only per-store address arithmetic is one add on the running byte offset
       const int col = tile.n0 + wn * 64 + l16 * 4;
       if (col < N) {
-        _Float16* C = (_Float16*)args.C + (size_t)tile.grp * N + col;
-        half4 bias4;
-        const bool has_bias = args.bias[tile.grp] != nullptr;
-        if (has_bias) bias4 = *reinterpret_cast<const half4*>((const _Float16*)args.bias[tile.grp] + col);
+        const __amdgpu_buffer_rsrc_t rc =
+            __builtin_amdgcn_make_buffer_rsrc(args.C, 0, (int)((uint32_t)rows * (uint32_t)args.ldc * 2u), 0x00020000);
+        const uint32_t row_bytes = (uint32_t)args.ldc * 2u;
+        uint32_t voff = ((uint32_t)(tile.m0 + wm * 128 + g * 4) * (uint32_t)args.ldc + (uint32_t)(tile.grp * N + col)) * 2u;
+        auto store_all = [&](auto with_bias, half4 bias4) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+          for (int i = 0; i < 8; ++i) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int row = tile.m0 + wm * 128 + i * 16 + g * 4 + r;
-            if (row < rows) {
+            for (int r = 0; r < 4; ++r) {
               half4 o;
 #pragma unroll
               for (int j = 0; j < 4; ++j) o[j] = f2h(acc[i][j][r]);
-              if (has_bias) o = o + bias4;     // half add on the rounded product, as the reference's next kernel does
-              __builtin_nontemporal_store(o, reinterpret_cast<half4*>(C + (size_t)row * args.ldc));
+              if (decltype(with_bias)::value) o = o + bias4;   // half add on the rounded product, as the reference's next kernel does
+              __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, o), rc, voff, 0, 2 /* nt */);
+              voff += row_bytes;
             }
+            voff += 12u * row_bytes;
           }
+        };
+        if (args.bias[tile.grp] != nullptr)
+          store_all(std::true_type{}, *reinterpret_cast<const half4*>((const _Float16*)args.bias[tile.grp] + col));
+        else
+          store_all(std::false_type{}, half4{});
       }
     }
     if (!has_next) break;
@@ -653,7 +663,7 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   if (t == DType::F16) {
     // few big tiles would leave most of the 256 CUs idle: fall back to 128-row tiles
     const long big = (long)((m_bound + 255) / 256) * ((n + 255) / 256) * g.groups;
-    if (big >= 128 && k >= 4 * kHBK)
+    if (big >= 128 && k >= 4 * kHBK && (uint64_t)m_bound * (uint64_t)ldc * 2u <= 0xffffffffull)
       launch_f16_persistent(a, stream);      // one workgroup per CU walks the tiles
     else
       launch_f16<4>(a, stream);              // few tiles: 128-row tiles spread over more CUs
