@@ -62,7 +62,7 @@ bool dtype_ok(et_dtype d) { return d == ET_FP32 || d == ET_FP16; }
 et::DType to_dt(et_dtype d) { return d == ET_FP32 ? et::DType::F32 : et::DType::F16; }
 
 struct LayerWs {
-  size_t qkv, ctx, attn, inter, seq, total;
+  size_t qkv, ctx, attn, inter, seq, wt, total;
 };
 
 LayerWs layer_ws(et_dtype dtype, int B, int S, int heads, int d) {
@@ -75,6 +75,8 @@ LayerWs layer_ws(et_dtype dtype, int B, int S, int heads, int d) {
   w.attn = off;  off += align_up(rows * H * e, 256);
   w.inter = off; off += align_up(rows * 4 * H * e, 256);
   w.seq = off;   off += align_up(((size_t)B + 1) * sizeof(int32_t), 256);
+  // fp16: k-contiguous copies of the six dense kernels (3 H^2 + H^2 + 4 H^2 + 4 H^2 elements) for the large-M GEMM
+  w.wt = off;    off += dtype == ET_FP16 ? align_up(12 * H * H * e, 256) : 0;
   w.total = off;
   return w;
 }
@@ -240,12 +242,35 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   int32_t* seq_start = (int32_t*)(base + ws.seq);
 
   et::launch_seq_start(batch_idx, T, rows, B, seq_start, st);
+  // The large-M fp16 GEMM reads k-contiguous weights with fewer LDS instructions; for the wide projections that is
+  // worth a transposed copy in the workspace per call (the caller's weights stay as they are).
+  const bool t_qkv = et::gemm_prefers_transposed_b(dt, rows, 3 * H, H, H, 3);
+  const bool t_o = et::gemm_prefers_transposed_b(dt, rows, H, H, H, 1);
+  const bool t_up = et::gemm_prefers_transposed_b(dt, rows, F, F, H, 1);
+  const bool t_down = et::gemm_prefers_transposed_b(dt, rows, H, H, F, 1);
+  char* wt = base + ws.wt;
+  const size_t HH = (size_t)H * H * e;
+  void* wt_q = wt; void* wt_k = wt + HH; void* wt_v = wt + 2 * HH; void* wt_o = wt + 3 * HH;
+  void* wt_up = wt + 4 * HH; void* wt_down = wt + 8 * HH;
+  {
+    et::TransposeJobs jobs;
+    if (t_qkv) {
+      jobs.add(w->attr_kernel_Q, wt_q, H, H);
+      jobs.add(w->attr_kernel_K, wt_k, H, H);
+      jobs.add(w->attr_kernel_V, wt_v, H, H);
+    }
+    if (t_o) jobs.add(w->attr_output_kernel, wt_o, H, H);
+    if (t_up) jobs.add(w->inter_kernel, wt_up, H, F);
+    if (t_down) jobs.add(w->output_kernel, wt_down, F, H);
+    et::launch_transpose_weights(jobs, st);
+  }
   // Q = from.Wq + bq, K = to.Wk + bk, V = to.Wv + bv into one [T,3H] buffer (bert_transformer_op.cu.cc:105-156)
   et::GemmGroups g3;
   g3.groups = 3;
   g3.A[0] = from_tensor; g3.A[1] = to_tensor; g3.A[2] = to_tensor;
-  g3.B[0] = w->attr_kernel_Q; g3.B[1] = w->attr_kernel_K; g3.B[2] = w->attr_kernel_V;
+  g3.B[0] = t_qkv ? wt_q : w->attr_kernel_Q; g3.B[1] = t_qkv ? wt_k : w->attr_kernel_K; g3.B[2] = t_qkv ? wt_v : w->attr_kernel_V;
   g3.bias[0] = w->attr_bias_Q; g3.bias[1] = w->attr_bias_K; g3.bias[2] = w->attr_bias_V;
+  g3.b_transposed = t_qkv;
   et::launch_gemm(dt, g3, qkv, 3 * H, rows, H, H, T, st);
   if ((s = check_launch(h, "QKV projection")) != ET_OK) return s;
   // QK^T, softmax, PV, un-pad (:159-192)
@@ -255,18 +280,21 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   // attention output projection + bias + residual(from_tensor) + LayerNorm (:195-213)
   et::GemmGroups g1;
   g1.groups = 1;
-  g1.A[0] = ctx; g1.B[0] = w->attr_output_kernel; g1.bias[0] = nullptr;
+  g1.A[0] = ctx; g1.B[0] = t_o ? wt_o : w->attr_output_kernel; g1.bias[0] = nullptr;
+  g1.b_transposed = t_o;
   et::launch_gemm(dt, g1, attn, H, rows, H, H, T, st);
   et::launch_bias_residual_layernorm(dt, attn, from_tensor, w->attr_output_bias, w->attr_output_layernorm_gamma,
                                      w->attr_output_layernorm_beta, rows, H, T, st);
   if ((s = check_launch(h, "attention output")) != ET_OK) return s;
   // FFN up + bias + GELU (:215-227)
-  g1.A[0] = attn; g1.B[0] = w->inter_kernel;
+  g1.A[0] = attn; g1.B[0] = t_up ? wt_up : w->inter_kernel;
+  g1.b_transposed = t_up;
   et::launch_gemm(dt, g1, inter, F, rows, F, H, T, st);
   et::launch_bias_gelu(dt, inter, w->inter_bias, rows, F, T, st);
   if ((s = check_launch(h, "FFN up")) != ET_OK) return s;
   // FFN down + bias + residual(LN1 output) + LayerNorm (:229-247)
-  g1.A[0] = inter; g1.B[0] = w->output_kernel;
+  g1.A[0] = inter; g1.B[0] = t_down ? wt_down : w->output_kernel;
+  g1.b_transposed = t_down;
   et::launch_gemm(dt, g1, out, H, rows, H, F, T, st);
   et::launch_bias_residual_layernorm(dt, out, attn, w->output_bias, w->output_layernorm_gamma,
                                      w->output_layernorm_beta, rows, H, T, st);
@@ -465,6 +493,38 @@ et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, voi
   g.A[0] = A; g.B[0] = B; g.bias[0] = bias;
   et::launch_gemm(to_dt(dtype), g, C, n, m, n, k, m_dev, (hipStream_t)stream);
   return check_launch(h, "gemm");
+}
+
+et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void* dst, int k, int n, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype == ET_FP16, "dtype must be ET_FP16");
+  ET_REQUIRE(h, src && dst && src != dst, "null or aliased tensor pointer");
+  ET_REQUIRE(h, k >= 1 && n >= 1 && k % 8 == 0 && n % 8 == 0, "k and n must be positive multiples of 8");
+  et::TransposeJobs jobs;
+  jobs.add(src, dst, k, n);
+  et::launch_transpose_weights(jobs, (hipStream_t)stream);
+  return check_launch(h, "weight transpose");
+}
+
+et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias, int m, int n,
+                     int k, const int32_t* m_dev, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype == ET_FP16, "dtype must be ET_FP16");
+  ET_REQUIRE(h, A && Bt && C, "null tensor pointer");
+  ET_REQUIRE(h, m >= 0 && n >= 1 && k >= 1, "bad dimensions");
+  if ((uint64_t)m * k * 2 > 0xffffffffull) return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
+  if (!et::gemm_takes_transposed_b(et::DType::F16, m, n, n, k, 1))
+    return fail(h, ET_UNSUPPORTED, "et_gemm_bt needs k % 32 == 0, n % 8 == 0 and at least 128 tiles of 256x256");
+  et::GemmGroups g;
+  g.groups = 1;
+  g.A[0] = A; g.B[0] = Bt; g.bias[0] = bias;
+  g.b_transposed = true;
+  et::launch_gemm(et::DType::F16, g, C, n, m, n, k, m_dev, (hipStream_t)stream);
+  return check_launch(h, "gemm_bt");
 }
 
 }  // extern "C"

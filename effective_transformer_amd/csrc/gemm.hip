@@ -34,6 +34,7 @@ struct GemmArgs {
   int ldc, m_bound, n, k, groups;
   int tiles_m, tiles_n;      // tiles_n per group
   int per_xcd;               // workgroups per XCD slot of the launch
+  int reverse_walk = 0;      // persistent kernel: walk the tiles from the last one
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -279,6 +280,7 @@ struct PTile {
   int m0, n0, grp;
 };
 
+template <bool BT>
 __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -303,6 +305,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
   auto valid = [&](int idx) { return idx / kXcds < per_xcd && tile_id(idx) < total; };
   auto locate = [&](int tile) {
     PTile t;
+    if (args.reverse_walk) tile = total - 1 - tile;
     const int tm = tile / tiles_n_all;
     const int tn_all = tile - tm * tiles_n_all;
     t.grp = tn_all / args.tiles_n;
@@ -326,10 +329,17 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
       const int row = q * 16 + (lane >> 2);
       const int c = (lane & 3) ^ a_swizzle(row);
       s.off[j] = ((uint32_t)(t.m0 + row) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
-      const int kr = q * 2 + (lane >> 5);
-      const int pc = ((lane & 31) - 8 * ((kr >> 3) & 1)) & 31;   // B rows 8..15, 24..31 are rotated by 128 bytes in LDS
-      const int col = min(t.n0 + pc * 8, N - 8);                 // columns beyond N: a valid column, never stored
-      s.off[2 + j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
+      if (BT) {
+        // B^T rows are columns of C.  LDS row j*16+l of a 64-column group holds column 4*l+j, so that the operand
+        // reads look like A's and a lane still owns 4 consecutive columns of C
+        const int col = min(t.n0 + (row & ~63) + (row & 15) * 4 + ((row >> 4) & 3), N - 1);   // beyond N: never stored
+        s.off[2 + j] = ((uint32_t)col * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+      } else {
+        const int kr = q * 2 + (lane >> 5);
+        const int pc = ((lane & 31) - 8 * ((kr >> 3) & 1)) & 31;   // B rows 8..15, 24..31 are rotated by 128 bytes in LDS
+        const int col = min(t.n0 + pc * 8, N - 8);                 // columns beyond N: a valid column, never stored
+        s.off[2 + j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
+      }
     }
     return s;
   };
@@ -343,7 +353,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
 #pragma unroll
     for (int j = 0; j < 2; ++j)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, ET_LDS_PTR(st + kPABytes + (wave * 2 + j) * 1024), 16, s.off[2 + j],
-                                               kt * kHBK * N * 2, 0, 0);
+                                               BT ? kt * kHBK * 2 : kt * kHBK * N * 2, 0, 0);
   };
 
   // LDS operand addresses: A row (wm*128 + i*16 + l16), chunk g (swizzled); B k-row g*8+kk, 4 columns
@@ -354,6 +364,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
     const int row = g * 8 + kk;
     b_rd[kk] = row * 512 + (((wn * 64 + l16 * 4) * 2 + 128 * ((row >> 3) & 1)) & 511);
   }
+  const int bt_rd = ((wn * 64 + l16) * 4 + (g ^ a_swizzle(l16))) * 16;   // B^T: row (wn*64 + j*16 + l16), chunk g
 
   int idx = blockIdx.x;
   if (!valid(idx)) return;
@@ -367,21 +378,28 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
   auto fetch_phase = [&](int kt_issue, const Src& s, bool check) {
     issue((u + 3) & 3, kt_issue, s);
     const unsigned char* st = smem + (u & 3) * kPStage;
-    uint2v raw[8];
+    if constexpr (BT) {
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint2v*>(st + kPABytes + b_rd[kk]);
+      for (int j = 0; j < 4; ++j) bop[j] = *reinterpret_cast<const half8*>(st + kPABytes + bt_rd + j * 16 * 64);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
+      for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
+    } else {
+      uint2v raw[8];
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {           // 8(k) x 4(n) block -> 4 operands
-      uint4v lo, hi;
+      for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint2v*>(st + kPABytes + b_rd[kk]);
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        lo[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x05040100u);
-        hi[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x07060302u);
+      for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {           // 8(k) x 4(n) block -> 4 operands
+        uint4v lo, hi;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          lo[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x05040100u);
+          hi[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x07060302u);
+        }
+        bop[2 * jj] = __builtin_bit_cast(half8, lo);
+        bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
       }
-      bop[2 * jj] = __builtin_bit_cast(half8, lo);
-      bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
     }
     if (check) wait_vmcnt<8>();                // this wave's share of k-step u+1 has landed (u+2, u+3 may fly)
     wait_lgkmcnt0();
@@ -620,10 +638,11 @@ int device_cu_count() {
   return cus;
 }
 
+template <bool BT>
 void launch_f16_persistent(GemmArgs a, hipStream_t stream) {
   static bool attr_set = false;
   if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_persistent_kernel),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_persistent_kernel<BT>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kPSmem);
     attr_set = true;
   }
@@ -633,10 +652,84 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream) {
   int grid = std::min(device_cu_count(), total);
   grid = (grid + kXcds - 1) / kXcds * kXcds;
   a.per_xcd = 0;     // derived on the device from the valid row count
-  gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
+  // k > n: A is the big operand and was written front to back by the kernel before this one, so its last rows are the
+  // ones most likely still in the last-level cache: walk the tiles from the end
+  a.reverse_walk = a.k > a.n ? 1 : 0;
+  gemm_f16_persistent_kernel<BT><<<grid, kPThreads, kPSmem, stream>>>(a);
+}
+
+// few big tiles would leave most of the 256 CUs idle: the persistent 256x256 kernel only runs when there is work
+// for at least half of them; C is addressed with 32-bit byte offsets there
+bool use_persistent(int m_bound, int ldc, int n, int k, int groups) {
+  const long big = (long)((m_bound + 255) / 256) * ((n + 255) / 256) * groups;
+  return big >= 128 && k >= 4 * kHBK && (uint64_t)m_bound * (uint64_t)ldc * 2u <= 0xffffffffull;
+}
+
+// ------------------------------------------------------------------------------------------
+// [k][n] -> [n][k] for fp16 weights: 64x64 tiles through LDS, 16-byte accesses on both sides.
+// ------------------------------------------------------------------------------------------
+struct TransposeArgs {
+  TransposeJobs jobs;
+  int tile_begin[TransposeJobs::kMax + 1];
+};
+constexpr int kTrTile = 64;
+constexpr int kTrStride = kTrTile + 8;    // halves; 144-byte rows keep the 16-byte row reads aligned
+
+__global__ __launch_bounds__(256) void transpose_weights_kernel(TransposeArgs args) {
+  __shared__ __attribute__((aligned(16))) _Float16 tile[kTrTile * kTrStride];
+  int job = 0;
+  while (job + 1 < args.jobs.count && (int)blockIdx.x >= args.tile_begin[job + 1]) ++job;
+  const int K = args.jobs.k[job], N = args.jobs.n[job];
+  const int tiles_n = (N + kTrTile - 1) / kTrTile;
+  const int t = blockIdx.x - args.tile_begin[job];
+  const int k0 = (t / tiles_n) * kTrTile, n0 = (t % tiles_n) * kTrTile;
+  const _Float16* __restrict__ src = (const _Float16*)args.jobs.src[job];
+  _Float16* __restrict__ dst = (_Float16*)args.jobs.dst[job];
+  // 64 rows x 8 chunks of 8 halves: two chunks per thread
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = threadIdx.x + u * 256;
+    const int r = i >> 3, c = i & 7;                  // source row k0+r, columns n0 + 8c ..
+    half8 v = {};
+    if (k0 + r < K && n0 + c * 8 < N) v = *reinterpret_cast<const half8*>(src + (size_t)(k0 + r) * N + n0 + c * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tile[(c * 8 + j) * kTrStride + r] = v[j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = threadIdx.x + u * 256;
+    const int r = i >> 3, c = i & 7;                  // destination row n0+r, columns k0 + 8c ..
+    if (n0 + r < N && k0 + c * 8 < K)
+      *reinterpret_cast<half8*>(dst + (size_t)(n0 + r) * K + k0 + c * 8) =
+          *reinterpret_cast<const half8*>(tile + r * kTrStride + c * 8);
+  }
 }
 
 }  // namespace
+
+bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
+  return t == DType::F16 && gemm_supported(t, n, k, groups) && k % 8 == 0 && use_persistent(m_bound, ldc, n, k, groups);
+}
+
+// Inside the layer the transposed copy pays off for the wide projections (QKV, FFN up: many column tiles re-read a
+// short k extent); with k > n the [k][n] rows of 512 contiguous bytes are the better fetch and the copy is skipped.
+bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
+  return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && (long)n * groups >= 2L * k;
+}
+
+void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream) {
+  if (jobs.count == 0) return;
+  TransposeArgs a;
+  a.jobs = jobs;
+  int total = 0;
+  for (int j = 0; j < jobs.count; ++j) {
+    a.tile_begin[j] = total;
+    total += ((jobs.k[j] + kTrTile - 1) / kTrTile) * ((jobs.n[j] + kTrTile - 1) / kTrTile);
+  }
+  for (int j = jobs.count; j <= TransposeJobs::kMax; ++j) a.tile_begin[j] = total;
+  transpose_weights_kernel<<<total, 256, 0, stream>>>(a);
+}
 
 bool gemm_supported(DType t, int n, int k, int groups) {
   if (groups < 1 || groups > 3 || n <= 0 || k <= 0) return false;
@@ -661,12 +754,12 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.k = k;
   a.groups = g.groups;
   if (t == DType::F16) {
-    // few big tiles would leave most of the 256 CUs idle: fall back to 128-row tiles
-    const long big = (long)((m_bound + 255) / 256) * ((n + 255) / 256) * g.groups;
-    if (big >= 128 && k >= 4 * kHBK && (uint64_t)m_bound * (uint64_t)ldc * 2u <= 0xffffffffull)
-      launch_f16_persistent(a, stream);      // one workgroup per CU walks the tiles
-    else
-      launch_f16<4>(a, stream);              // few tiles: 128-row tiles spread over more CUs
+    if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
+      if (g.b_transposed) launch_f16_persistent<true>(a, stream);
+      else launch_f16_persistent<false>(a, stream);
+    } else {
+      launch_f16<4>(a, stream);                             // few tiles: 128-row tiles spread over more CUs
+    }
   } else {
     a.tiles_m = (m_bound + kFBM - 1) / kFBM;
     a.tiles_n = (n + kFBN - 1) / kFBN;

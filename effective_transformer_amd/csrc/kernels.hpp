@@ -69,8 +69,26 @@ struct GemmGroups {
   const void* B[3];
   const void* bias[3];
   int groups;
+  // true: B[g] holds the transpose, [n][k] row-major (see launch_transpose_weights); only where
+  // gemm_takes_transposed_b() says so
+  bool b_transposed = false;
 };
 bool gemm_supported(DType t, int n, int k, int groups);
+// The large-M fp16 kernel is faster when B comes k-contiguous ([n][k]): both operands then reach the
+// MFMA with 128-bit LDS reads and no register transpose.  True when launch_gemm would use that kernel.
+bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
+// ... and where the encoder layer found the extra copy worth its time (measured inside the layer, not in isolation).
+bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
+// dst[j] ([n][k], row-major) = transpose of src[j] ([k][n], row-major), fp16, one launch for all jobs.
+struct TransposeJobs {
+  static constexpr int kMax = 6;
+  const void* src[kMax];
+  void* dst[kMax];
+  int k[kMax], n[kMax];
+  int count = 0;
+  void add(const void* s, void* d, int k_, int n_) { src[count] = s; dst[count] = d; k[count] = k_; n[count] = n_; ++count; }
+};
+void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream);
 void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k,
                  const int32_t* rows_dev, hipStream_t stream);
 

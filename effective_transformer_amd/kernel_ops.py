@@ -107,3 +107,24 @@ def gemm(a, b, bias=None, m: Optional[int] = None, m_dev: Optional[torch.Tensor]
     _call("et_gemm", a.device, _dtype_code(a.dtype), _p(a), _p(b), _p(out), _p(bias), rows if m is None else m, n, k,
           _p(m_dev), _stream())
     return out
+
+
+def transpose_weight(w, out: Optional[torch.Tensor] = None):
+    """[k, n] -> [n, k] (fp16), the layout gemm_bt takes."""
+    k, n = w.shape
+    if out is None:
+        out = torch.empty(n, k, dtype=w.dtype, device=w.device)
+    _call("et_transpose_weight", w.device, _dtype_code(w.dtype), _p(w), _p(out), k, n, _stream())
+    return out
+
+
+def gemm_bt(a, bt, bias=None, m: Optional[int] = None, m_dev: Optional[torch.Tensor] = None,
+            out: Optional[torch.Tensor] = None):
+    """a [m, k] . bt [n, k]^T: the large-M kernel of the encoder layer."""
+    rows, k = a.shape
+    n = bt.shape[0]
+    if out is None:
+        out = torch.zeros(rows, n, dtype=a.dtype, device=a.device)
+    _call("et_gemm_bt", a.device, _dtype_code(a.dtype), _p(a), _p(bt), _p(out), _p(bias), rows if m is None else m, n,
+          k, _p(m_dev), _stream())
+    return out

@@ -193,6 +193,16 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
 et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias,
                   int m, int n, int k, const int32_t* m_dev, void* stream);
 
+/* dst[n][k] = transpose of src[k][n] (both row-major), fp16 only.  No counterpart in the reference, which hands the
+ * TF dense kernels [in,out] to cuBLAS as they are; et_layer does this internally for its large-M GEMMs. */
+et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void* dst, int k, int n, void* stream);
+
+/* et_gemm with the second operand k-contiguous: C[m,n] = A[m,k] . Bt[n,k]^T (+ bias), fp16 only.  This is the kernel
+ * et_layer runs once a batch has enough tokens to fill the chip (same cublasGemmEx call sites as et_gemm);
+ * ET_UNSUPPORTED for shapes with fewer than 128 tiles of 256x256, which go through et_gemm's kernels. */
+et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
+                     int m, int n, int k, const int32_t* m_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -316,3 +316,34 @@ def test_gemm(k, dtype, m, n, k_):
         md = torch.tensor([m - 5], dtype=torch.int32, device="cuda")
         got2 = k.gemm(dev(a), dev(b), m_dev=md).cpu().numpy()
         assert np.array_equal(got2[:m - 5], got[:m - 5]) and np.all(got2[m - 5:] == 0)
+
+
+# The k-contiguous-B kernel only runs from 128 tiles of 256x256 on: shapes are sized for that, the
+# oracle product is taken on the CPU in float64 for a sample of rows.
+@pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072)])
+def test_gemm_bt(k, m, n, k_):
+    print("gemm_bt", m, n, k_, flush=True)
+    rng = np.random.RandomState(m + n + k_)
+    a = o.rnd(rng.randn(m, k_), "fp16")
+    b = o.rnd(0.05 * rng.randn(k_, n), "fp16")
+    bias = o.rnd(rng.randn(n), "fp16")
+    bt = k.transpose_weight(dev(b))
+    assert np.array_equal(bt.cpu().numpy(), b.T)                       # the transpose is a pure copy
+    got = k.gemm_bt(dev(a), bt).cpu().numpy()
+    # the same rows through the untransposed kernel: both accumulate k in the same order
+    assert np.array_equal(got, k.gemm(dev(a), dev(b)).cpu().numpy())
+    rows = np.unique(np.concatenate([np.arange(0, 300), np.arange(m - 300, m), rng.randint(0, m, 400)]))
+    exact = a[rows].astype(np.float64) @ b.astype(np.float64)
+    assert np.all(np.abs(got[rows].astype(np.float64) - exact) <= 0.51 * half_ulp(exact) + 1e-5 * np.abs(exact).max())
+    gotb = k.gemm_bt(dev(a), bt, bias=dev(bias)).cpu().numpy()
+    assert np.array_equal(gotb, o.hadd(got, bias))
+    md = torch.tensor([m - 301], dtype=torch.int32, device="cuda")
+    got2 = k.gemm_bt(dev(a), bt, m_dev=md).cpu().numpy()
+    assert np.array_equal(got2[:m - 301], got[:m - 301]) and np.all(got2[m - 301:] == 0)
+
+
+def test_gemm_bt_small_shapes_are_refused(k):
+    a = torch.zeros(1000, 768, dtype=torch.float16, device="cuda")
+    bt = torch.zeros(768, 768, dtype=torch.float16, device="cuda")
+    with pytest.raises(Exception, match="128 tiles"):
+        k.gemm_bt(a, bt)
