@@ -20,11 +20,13 @@ if ROOT not in sys.path:
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (FETCH_SIZE scaled by 2.0, the factor a
 # plain device copy of known size shows in the same run); cfg3 shapes.  (read + write) in bytes.
 MEASURED_TRAFFIC = {
-    ("cfg3", "gemm_ffn_up"): (369.1 + 236.7) * (1 << 20),
-    ("cfg3", "gemm_qkv"): (234.3 + 177.5) * (1 << 20),
+    ("cfg3", "gemm_ffn_up"): (376.6 + 237.3) * (1 << 20),
+    ("cfg3", "gemm_ffn_down"): (327.4 + 59.2) * (1 << 20),
+    ("cfg3", "gemm_qkv"): (241.8 + 178.1) * (1 << 20),
+    ("cfg3", "gemm_attn_out"): (86.2 + 59.3) * (1 << 20),
     ("cfg3", "bias_gelu"): (236.8 + 236.7) * (1 << 20),
-    ("cfg3", "bias_residual_layernorm"): (118.5 + 59.2) * (1 << 20),
-    ("cfg3", "attention"): (226.3 + 59.2) * (1 << 20),
+    ("cfg3", "bias_residual_layernorm"): (118.4 + 59.2) * (1 << 20),
+    ("cfg3", "attention"): (202.2 + 59.2) * (1 << 20),
 }
 # ms/batch the reference publishes for the same model/batch/sequence recipe (Tesla V100, Readme.md:65-89 of the
 # reference); vs_baseline = published ms / measured ms.
