@@ -169,6 +169,9 @@ template <typename T> struct AttnCfg;
 template <> struct AttnCfg<_Float16> {
   static constexpr int kQkStride = kD + 8;   // halves; 144-byte rows keep 16-byte reads of 8 consecutive rows on distinct banks
   static constexpr int kVtPad = 4;           // halves
+  // fp16 keeps V row-major ([key][feature]) and transposes 8x4 blocks in registers: 160-byte rows put the four
+  // key groups of an 8-byte operand read 128 bytes apart modulo the 256-byte bank span
+  static constexpr int kVStride = kD + 16;
 };
 template <> struct AttnCfg<float> {
   static constexpr int kQkStride = kD + 4;   // floats; 272-byte rows
@@ -180,7 +183,7 @@ struct AttnSmem {
   static constexpr int kSp = NKT * 16;
   static constexpr int kVtStride = kSp + AttnCfg<T>::kVtPad;
   static constexpr size_t kQBytes = (size_t)kSp * AttnCfg<T>::kQkStride * sizeof(T);
-  static constexpr size_t kVtBytes = (size_t)kD * kVtStride * sizeof(T);
+  static constexpr size_t kVtBytes = sizeof(T) == 2 ? (size_t)kSp * (kD + 16) * sizeof(T) : (size_t)kD * kVtStride * sizeof(T);
   static constexpr size_t kBytes = 2 * kQBytes + kVtBytes + kSp * sizeof(int);
 };
 
@@ -207,6 +210,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   using C = Chunk16<T>;
   constexpr int kQS = Cfg::kQkStride;
   constexpr int kVS = Sm::kVtStride;
+  constexpr int kVR = kD + 16;                // fp16: stride of the row-major V tile (AttnCfg<_Float16>::kVStride)
   constexpr int kSp = Sm::kSp;
   constexpr int kCpr = kD / C::kElems;       // 16-byte chunks per head row
   constexpr int QPW = NKT > 4 ? NKT / 4 : 1; // query tiles per wavefront
@@ -298,8 +302,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
       if (tok_of_pos[pos] < 0) {
         if (sizeof(T) == 2) {
           reinterpret_cast<uint32_t*>(Ks + pos * kQS)[w] = 0u;                // 2 halves
-          Vt[(2 * w) * kVS + pos] = (T)0;
-          Vt[(2 * w + 1) * kVS + pos] = (T)0;
+          reinterpret_cast<uint32_t*>(Vt + pos * kVR)[w] = 0u;                // V is row-major for fp16
         } else {
           Ks[pos * kQS + 2 * w] = (T)0; Ks[pos * kQS + 2 * w + 1] = (T)0;
           Vt[(2 * w) * kVS + pos] = (T)0;
@@ -319,8 +322,12 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
         const int c = my_c[k];
         *reinterpret_cast<V16*>(Qs + pos * kQS + c * C::kElems) = rq[k];
         *reinterpret_cast<V16*>(Ks + pos * kQS + c * C::kElems) = rk[k];
+        if constexpr (sizeof(T) == 2) {
+          *reinterpret_cast<V16*>(Vt + pos * kVR + c * C::kElems) = rv[k];
+        } else {
 #pragma unroll
-        for (int j = 0; j < C::kElems; ++j) Vt[(c * C::kElems + j) * kVS + pos] = rv[k][j];
+          for (int j = 0; j < C::kElems; ++j) Vt[(c * C::kElems + j) * kVS + pos] = rv[k][j];
+        }
       }
     }
     __syncthreads();
@@ -409,6 +416,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
       if constexpr (sizeof(T) == 2) {
+        // A operand j = V^T rows {4*l + j}: the lane reads 4 consecutive features of its 8 keys (the keys its
+        // probability registers belong to) and transposes the 8x4 block with v_perm_b32
 #pragma unroll
         for (int ks = 0; ks < NKT / 2; ++ks) {
           if (2 * ks < n_tiles) {
@@ -418,18 +427,24 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
               p[r] = f2h(s[2 * ks][r]);
               p[4 + r] = f2h(s[2 * ks + 1][r]);
             }
+            typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            u2 raw[8];
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt) {
-              const T* vrow = Vt + (dt * 16 + l16) * kVS + ks * 32 + g * 4;
-              const half4 lo = *reinterpret_cast<const half4*>(vrow);
-              const half4 hi = *reinterpret_cast<const half4*>(vrow + 16);
-              half8 a;
+            for (int kk = 0; kk < 8; ++kk) {
+              const int key = ks * 32 + (kk >> 2) * 16 + g * 4 + (kk & 3);
+              raw[kk] = *reinterpret_cast<const u2*>(Vt + key * kVR + l16 * 4);
+            }
 #pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                a[r] = lo[r];
-                a[4 + r] = hi[r];
+            for (int jj = 0; jj < 2; ++jj) {
+              u4 lo, hi;
+#pragma unroll
+              for (int q4 = 0; q4 < 4; ++q4) {
+                lo[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x05040100u);
+                hi[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x07060302u);
               }
-              o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, p, o[dt], 0, 0, 0);
+              o[2 * jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, lo), p, o[2 * jj], 0, 0, 0);
+              o[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, hi), p, o[2 * jj + 1], 0, 0, 0);
             }
           }
         }
@@ -447,17 +462,32 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
           }
         }
       }
-      // ---- write the lane's 4x4 features of its query's packed row --------------------------
+      // ---- write the lane's 16 features of its query's packed row --------------------------
       const int tq = tok_of_pos[q];
       if (tq >= 0) {
-        T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+        if constexpr (sizeof(T) == 2) {
+          // o[j][r] is feature 16*g + 4*r + j: 16 consecutive features
+          half8 v0, v1;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          typedef T out4 __attribute__((ext_vector_type(4)));
-          out4 v;
+          for (int r = 0; r < 2; ++r)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = (T)o[dt][r];
-          *reinterpret_cast<out4*>(orow + dt * 16) = v;
+            for (int j = 0; j < 4; ++j) {
+              v0[4 * r + j] = f2h(o[j][r]);
+              v1[4 * r + j] = f2h(o[j][2 + r]);
+            }
+          T* orow = dst + (size_t)tq * H + head * kD + g * 16;
+          *reinterpret_cast<half8*>(orow) = v0;
+          *reinterpret_cast<half8*>(orow + 8) = v1;
+        } else {
+          T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) {
+            typedef T out4 __attribute__((ext_vector_type(4)));
+            out4 v;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = (T)o[dt][r];
+            *reinterpret_cast<out4*>(orow + dt * 16) = v;
+          }
         }
       }
     }

@@ -7,6 +7,8 @@
 // All of it is HBM-bound byte and integer work: the scan runs on 64-lane DPP prefix sums, the
 // row movers use one 128-bit access per lane on a flattened (row, 16-byte chunk) index space so
 // that every lane of every wavefront carries data.
+#include <type_traits>
+
 #include "et_device.hpp"
 #include "kernels.hpp"
 
@@ -65,15 +67,21 @@ __global__ __launch_bounds__(kScanThreads) void scan_index_kernel(const int32_t*
     // few tiles: add up everything in front of this tile straight from the input (it sits in L2), saving a launch
     const int n4 = blockIdx.x * tile / 4;             // int4 words in front of this tile (tile is a multiple of 4)
     const int4* in4 = reinterpret_cast<const int4*>(in);
-    constexpr int kU = 8;                             // independent loads in flight per thread
     int i = threadIdx.x;
-    for (; i + (kU - 1) * kScanThreads < n4; i += kU * kScanThreads) {
-      int4 v[kU];
+    // 32, then 8 independent loads in flight per thread: the longest front (252 KB at 64K positions) is two round
+    // trips to L2 instead of one per 4 KB
+    auto batch = [&](auto ku) {
+      constexpr int kU = decltype(ku)::value;
+      for (; i + (kU - 1) * kScanThreads < n4; i += kU * kScanThreads) {
+        int4 v[kU];
 #pragma unroll
-      for (int u = 0; u < kU; ++u) v[u] = in4[i + u * kScanThreads];
+        for (int u = 0; u < kU; ++u) v[u] = in4[i + u * kScanThreads];
 #pragma unroll
-      for (int u = 0; u < kU; ++u) part += v[u].x + v[u].y + v[u].z + v[u].w;
-    }
+        for (int u = 0; u < kU; ++u) part += v[u].x + v[u].y + v[u].z + v[u].w;
+      }
+    };
+    batch(std::integral_constant<int, 32>{});
+    batch(std::integral_constant<int, 8>{});
     for (; i < n4; i += kScanThreads) {
       const int4 v = in4[i];
       part += v.x + v.y + v.z + v.w;
