@@ -286,6 +286,16 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   const int last_pos = min(max(last_pos_raw, 0), seq_len - 1);
   const int n_tiles = last_pos / 16 + 1;    // 16-row tiles that hold at least one token (queries and keys)
 
+  // mask value -> additive bias, once for all heads: (1 - m) * -10000 in float as the reference computes it, kept in
+  // the element type (exact for 0/1 masks); keys beyond seq_len do not exist
+#pragma unroll
+  for (int qi = 0; qi < QPW; ++qi)
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        mreg[qi][kt][r] = kt * 16 + g * 4 + r < seq_len ? (T)((1.0f - (float)mreg[qi][kt][r]) * -10000.0f) : (T)-INFINITY;
+
   // ---- position table, then zero the key / value slots that hold no token (once: heads only overwrite tokens) ----
   for (int i = threadIdx.x; i < kSp; i += kAttnThreads) tok_of_pos[i] = -1;
   __syncthreads();
@@ -384,25 +394,20 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
       // ---- masked softmax over the keys of query q ------------------------------------------
       float mx = 0.f;                          // clamp of the maximum at 0
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) {
-        const int key0 = kt * 16 + g * 4;
+      for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          // keys beyond seq_len do not exist
-          const float tv = key0 + r < seq_len
-                               ? s[kt][r] * scaler + (1.0f - (float)mreg[qi][kt][r]) * -10000.0f
-                               : -INFINITY;
+          const float tv = s[kt][r] * scaler + (float)mreg[qi][kt][r];   // mreg: (1 - mask) * -10000, -inf beyond seq_len
           s[kt][r] = tv;
           mx = fmaxf(mx, tv);
         }
-      }
-      mx = xor_lanes_16_32_max(mx);
+      mx = xor_lanes_16_32_max(mx) * kLog2e;
       float sum = 0.f;
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          s[kt][r] = __builtin_amdgcn_exp2f((s[kt][r] - mx) * kLog2e);
+          s[kt][r] = __builtin_amdgcn_exp2f(s[kt][r] * kLog2e - mx);
           sum += s[kt][r];
         }
       sum = xor_lanes_16_32_sum(sum) + 1e-6f;
