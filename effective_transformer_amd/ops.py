@@ -207,6 +207,15 @@ class EffectiveTransformerEncoder:
             LayerWeights.from_slots(self.device, dtype, weights_value[16 * l:16 * l + 16]) for l in range(num_layers)]
         self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor]] = {}
 
+    @classmethod
+    def from_checkpoint(cls, path: str, head_num: int, size_per_head: int, dtype: torch.dtype, device="cuda",
+                        num_layers: Optional[int] = None, prefix: Optional[str] = None):
+        """Encoder from a local `.npz` / `.safetensors` file with TF-BERT or Hugging Face tensor names
+        (see weights.py for the name map)."""
+        from . import weights as _weights
+        ws = _weights.load_weights(path, num_layers, prefix)
+        return cls(len(ws) // 16, head_num, size_per_head, ws, dtype, device)
+
     def __call__(self, from_tensor: torch.Tensor, input_mask: torch.Tensor, attention_mask: torch.Tensor,
                  sync_count: bool = True) -> torch.Tensor:
         B, S = input_mask.shape
