@@ -98,6 +98,21 @@ def per_kernel(wl, T, mask_np, iters=20):
     add("input_scan_compress", ms, "hbm", 2 * T * H * e + 4 * B * S + 8 * T + 4)
     ms = _time_kernel(run_output, iters)
     add("output_restore", ms, "hbm", T * H * e + B * S * H * e + 8 * T)
+    # the step in front of the path: BERT-base embedding block fused with the input op (ids -> packed rows)
+    V, Vt, Pmax = 30522, 2, 512
+    emb = ops.EmbeddingWeights(x.device, dt, rnd(V, H), rnd(H), rnd(H), token_type_embeddings=rnd(Vt, H),
+                               position_embeddings=rnd(Pmax, H))
+    ids = torch.randint(0, V, (B, S), dtype=torch.int32, device="cuda")
+    tts = torch.randint(0, Vt, (B, S), dtype=torch.int32, device="cuda")
+    to_e = torch.empty_like(x)
+
+    def run_embed():
+        _lib.check(lib.et_embedding_input(h, code, C.byref(emb.struct), P(ids), P(tts), P(mask), P(to_e), P(vwn), P(bidx),
+                                          P(widx), B, S, heads, d, P(ws), ws.numel(), st, None), h)
+
+    ms = _time_kernel(run_embed, iters)
+    add("embedding_input", ms, "hbm", 2 * T * H * e + 12 * B * S + 16 * T + 4)
+    run_input()      # leaves the index arrays of the activation path in place
     # row kernels
     a = rnd(T, H); r = rnd(T, H); bias = rnd(H); gam = rnd(H); bet = rnd(H)
     ms = _time_kernel(lambda: k.add_bias_input_layernorm(a, r, bias, gam, bet), iters)

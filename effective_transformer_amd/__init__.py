@@ -9,7 +9,8 @@ from . import _lib  # noqa: F401
 def __getattr__(name):
     # torch-facing API is imported lazily so that `import effective_transformer_amd` stays cheap
     if name in ("effective_transformer_input", "effective_transformer", "effective_transformer_output",
-                "get_sequence_output", "EffectiveTransformerEncoder", "GraphedEncoder", "LayerWeights", "handle"):
+                "get_sequence_output", "EffectiveTransformerEncoder", "GraphedEncoder", "LayerWeights", "handle",
+                "EmbeddingWeights", "effective_transformer_embedding_input"):
         from . import ops
         return getattr(ops, name)
     raise AttributeError(name)

@@ -28,6 +28,12 @@ class LayerWeights(C.Structure):
     _fields_ = [(name, C.c_void_p) for name in WEIGHT_FIELDS]
 
 
+class EmbeddingWeights(C.Structure):
+    _fields_ = [("word_embeddings", C.c_void_p), ("token_type_embeddings", C.c_void_p),
+                ("position_embeddings", C.c_void_p), ("layernorm_gamma", C.c_void_p), ("layernorm_beta", C.c_void_p),
+                ("vocab_size", C.c_int), ("type_vocab_size", C.c_int), ("max_position_embeddings", C.c_int)]
+
+
 class EtError(RuntimeError):
     def __init__(self, status: int, message: str):
         super().__init__("%s: %s" % (STATUS_NAMES.get(status, str(status)), message))
@@ -47,6 +53,8 @@ SIGNATURES = {
     "et_layer_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "et_seq_workspace_bytes": (_sz, [_i]),
     "et_input": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp, _ip]),
+    "et_embedding_input": (_i, [_vp, _i, C.POINTER(EmbeddingWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
+                                _vp, _sz, _vp, _ip]),
     "et_layer": (_i, [_vp, _i, C.POINTER(LayerWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                       _vp, _sz, _vp]),
     "et_output": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -195,6 +195,47 @@ et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const i
   return ET_OK;
 }
 
+et_status et_embedding_input(et_handle h, et_dtype dtype, const et_embedding_weights* emb, const int32_t* input_ids,
+                             const int32_t* token_type_ids, const int32_t* mask, void* to_tensor,
+                             int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx, int batch_size,
+                             int seq_len, int head_num, int size_per_head, void* workspace, size_t workspace_bytes,
+                             void* stream, int32_t* valid_word_num_host) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, emb != nullptr, "null embeddings");
+  ET_REQUIRE(h, emb->word_embeddings && emb->layernorm_gamma && emb->layernorm_beta, "null embedding table or LayerNorm weight");
+  ET_REQUIRE(h, emb->vocab_size >= 1, "vocab_size must be >= 1");
+  ET_REQUIRE(h, (emb->token_type_embeddings == nullptr) == (token_type_ids == nullptr),
+             "token_type_ids and token_type_embeddings go together");
+  ET_REQUIRE(h, emb->token_type_embeddings == nullptr || emb->type_vocab_size >= 1, "type_vocab_size must be >= 1");
+  ET_REQUIRE(h, emb->position_embeddings == nullptr || seq_len <= emb->max_position_embeddings,
+             "seq_len exceeds max_position_embeddings");
+  ET_REQUIRE(h, input_ids && mask && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  ET_REQUIRE(h, workspace != nullptr, "null workspace");
+  if (workspace_bytes < et_input_workspace_bytes(batch_size, seq_len))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "et_embedding_input needs et_input_workspace_bytes(batch_size, seq_len)");
+  const int H = head_num * size_per_head;
+  if (!et::bias_residual_layernorm_supported(to_dt(dtype), H))
+    return fail(h, ET_UNSUPPORTED, "hidden size not supported by the LayerNorm kernel");
+  hipStream_t st = (hipStream_t)stream;
+  et::launch_scan_index(mask, batch_size * seq_len, nullptr, batch_idx, word_idx, valid_word_num_dev, seq_len,
+                        (int32_t*)workspace, st);
+  if ((s = check_launch(h, "mask scan")) != ET_OK) return s;
+  et::launch_embed_layernorm(to_dt(dtype), to_tensor, input_ids, token_type_ids, batch_idx, word_idx,
+                             emb->word_embeddings, emb->vocab_size, emb->token_type_embeddings, emb->type_vocab_size,
+                             emb->position_embeddings, emb->max_position_embeddings, emb->layernorm_gamma,
+                             emb->layernorm_beta, batch_size * seq_len, H, seq_len, valid_word_num_dev, st);
+  if ((s = check_launch(h, "embedding")) != ET_OK) return s;
+  if (valid_word_num_host) {
+    ET_HIP(h, hipMemcpyAsync(valid_word_num_host, valid_word_num_dev, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    ET_HIP(h, hipStreamSynchronize(st));
+  }
+  return ET_OK;
+}
+
 et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const void* from_tensor,
                    const void* to_tensor, const void* attr_mask, const int32_t* valid_word_num_dev,
                    const int32_t* batch_idx, const int32_t* word_idx, void* out, int batch_size, int from_seq_len,

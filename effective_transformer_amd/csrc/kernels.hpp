@@ -44,6 +44,14 @@ void launch_bias_residual_layernorm(DType t, void* out, const void* input, const
                                     const void* gamma, const void* beta, int m, int n,
                                     const int32_t* rows_dev, hipStream_t stream);
 
+// out[t,:] = LayerNorm(word[ids[p]] + type[type_ids[p]] + pos[word_idx[t]]) * gamma + beta for packed row t at padded
+// position p = batch_idx[t]*seq_len + word_idx[t]; eps 1e-12.  type_ids/type_table and pos_table may be null.
+// n must satisfy bias_residual_layernorm_supported.
+void launch_embed_layernorm(DType t, void* out, const int32_t* ids, const int32_t* type_ids, const int32_t* batch_idx,
+                            const int32_t* word_idx, const void* word_table, int vocab, const void* type_table,
+                            int type_vocab, const void* pos_table, int max_pos, const void* gamma, const void* beta,
+                            int m, int n, int seq_len, const int32_t* rows_dev, hipStream_t stream);
+
 // ---- attention.hip -----------------------------------------------------------------------
 void launch_qkv_bias_pad(DType t, const void* Q, const void* bQ, const void* K, const void* bK,
                          const void* V, const void* bV, void* q_buf, void* k_buf, void* v_buf,

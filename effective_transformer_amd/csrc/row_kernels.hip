@@ -171,6 +171,93 @@ __global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Embedding lookup + post-processing written straight into the packed token matrix (reference graph:
+// sample/tensorflow/modeling.py:380-521): row t = LayerNorm(word[ids[p]] + type[type_ids[p]] + pos[s]) for the t-th
+// valid position p = (b, s).  One wavefront per packed row, same register-resident two-pass LayerNorm as above with
+// the TF layer_norm epsilon; ids outside a table read as a zero row (what tf.gather does on a GPU).
+// ------------------------------------------------------------------------------------------
+template <typename T, int VEC, int ITERS>
+__global__ __launch_bounds__(kLnThreads) void embed_layernorm_kernel(
+    T* __restrict__ out, const int32_t* __restrict__ ids, const int32_t* __restrict__ type_ids,
+    const int32_t* __restrict__ batch_idx, const int32_t* __restrict__ word_idx, const T* __restrict__ word_table,
+    int vocab, const T* __restrict__ type_table, int type_vocab, const T* __restrict__ pos_table, int max_pos,
+    const T* __restrict__ gamma, const T* __restrict__ beta, int m, int n, int seq_len,
+    const int32_t* __restrict__ rows_dev) {
+  using V = typename RowVec<T, VEC>::type;
+  const int rows = rows_dev ? min(*rows_dev, m) : m;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = blockIdx.x * kLnWaves + threadIdx.x / kWave;
+  const int nwaves = gridDim.x * kLnWaves;
+  const int vpr = n / VEC;
+
+  V g[ITERS], be[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = lane + i * kWave;
+    if (c < vpr) {
+      g[i] = reinterpret_cast<const V*>(gamma)[c];
+      be[i] = reinterpret_cast<const V*>(beta)[c];
+    }
+  }
+  const float inv_n = 1.0f / (float)n;
+
+  for (int r = wave; r < rows; r += nwaves) {
+    const int b = batch_idx[r], sp = word_idx[r];
+    const int p = b * seq_len + sp;
+    const int id = ids[p];
+    const int tt = type_ids ? type_ids[p] : 0;
+    const bool id_ok = id >= 0 && id < vocab;
+    const bool tt_ok = type_table != nullptr && tt >= 0 && tt < type_vocab;
+    const bool pos_ok = pos_table != nullptr && sp < max_pos;
+    const V* wrow = reinterpret_cast<const V*>(word_table + (size_t)(id_ok ? id : 0) * n);
+    const V* trow = reinterpret_cast<const V*>(type_table + (size_t)(tt_ok ? tt : 0) * n);
+    const V* prow = reinterpret_cast<const V*>(pos_table + (size_t)(pos_ok ? sp : 0) * n);
+    float x[ITERS][VEC];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+      V s;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s[j] = (T)0;
+      if (c < vpr) {
+        if (id_ok) s = wrow[c];
+        if (tt_ok) s = s + trow[c];             // element-type adds in the order of the graph: word, += type, += position
+        if (pos_ok) s = s + prow[c];
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        x[i][j] = c < vpr ? (float)s[j] : 0.f;
+        sum += x[i][j];
+      }
+    }
+    const float mean = wave_sum(sum) * inv_n;
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float dlt = x[i][j] - mean;
+        sq += c < vpr ? dlt * dlt : 0.f;
+      }
+    }
+    const float rstd = __builtin_amdgcn_rsqf(wave_sum(sq) * inv_n + 1e-12f);
+    V* orow = reinterpret_cast<V*>(out + (size_t)r * n);
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = lane + i * kWave;
+      if (c < vpr) {
+        V y;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) y[j] = (T)(((x[i][j] - mean) * rstd) * (float)g[i][j] + (float)be[i][j]);
+        orow[c] = y;
+      }
+    }
+  }
+}
+
 template <typename T>
 bool ln_pick(int n, int& vec, int& iters) {
   const int max_vec = 16 / (int)sizeof(T);
@@ -225,7 +312,64 @@ void ln_launch(void* out, const void* input, const void* bias, const void* gamma
     ln_launch_iters<T, MV / 4>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
 }
 
+struct EmbedArgs {
+  void* out;
+  const int32_t *ids, *type_ids, *batch_idx, *word_idx;
+  const void *word_table, *type_table, *pos_table, *gamma, *beta;
+  int vocab, type_vocab, max_pos, m, n, seq_len;
+  const int32_t* rows_dev;
+};
+
+template <typename T, int VEC>
+void embed_launch_iters(int iters, int grid, hipStream_t stream, const EmbedArgs& a) {
+#define ET_EMB_CASE(I)                                                                                              \
+  case I:                                                                                                           \
+    embed_layernorm_kernel<T, VEC, I><<<grid, kLnThreads, 0, stream>>>(                                             \
+        (T*)a.out, a.ids, a.type_ids, a.batch_idx, a.word_idx, (const T*)a.word_table, a.vocab,                     \
+        (const T*)a.type_table, a.type_vocab, (const T*)a.pos_table, a.max_pos, (const T*)a.gamma, (const T*)a.beta, \
+        a.m, a.n, a.seq_len, a.rows_dev);                                                                           \
+    break;
+  switch (iters) {
+    ET_EMB_CASE(1)
+    ET_EMB_CASE(2)
+    ET_EMB_CASE(3)
+    ET_EMB_CASE(4)
+    ET_EMB_CASE(5)
+    ET_EMB_CASE(6)
+    ET_EMB_CASE(7)
+    ET_EMB_CASE(8)
+  }
+#undef ET_EMB_CASE
+}
+
+template <typename T>
+void embed_launch(const EmbedArgs& a, hipStream_t stream) {
+  int vec = 0, iters = 0;
+  if (!ln_pick<T>(a.n, vec, iters)) return;
+  const int grid = (int)min((long)(a.m + kLnWaves - 1) / kLnWaves, 256L * 8);
+  constexpr int MV = 16 / (int)sizeof(T);
+  if (vec == MV)
+    embed_launch_iters<T, MV>(iters, grid, stream, a);
+  else if (vec == MV / 2)
+    embed_launch_iters<T, MV / 2>(iters, grid, stream, a);
+  else
+    embed_launch_iters<T, MV / 4>(iters, grid, stream, a);
+}
+
 }  // namespace
+
+void launch_embed_layernorm(DType t, void* out, const int32_t* ids, const int32_t* type_ids, const int32_t* batch_idx,
+                            const int32_t* word_idx, const void* word_table, int vocab, const void* type_table,
+                            int type_vocab, const void* pos_table, int max_pos, const void* gamma, const void* beta,
+                            int m, int n, int seq_len, const int32_t* rows_dev, hipStream_t stream) {
+  if (m <= 0) return;
+  EmbedArgs a{out, ids, type_ids, batch_idx, word_idx, word_table, type_table, pos_table, gamma, beta,
+              vocab, type_vocab, max_pos, m, n, seq_len, rows_dev};
+  if (t == DType::F32)
+    embed_launch<float>(a, stream);
+  else
+    embed_launch<_Float16>(a, stream);
+}
 
 bool bias_gelu_supported(DType t, int n) { return n > 0 && ((size_t)n * elem_size(t)) % 16 == 0; }
 

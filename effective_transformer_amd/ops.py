@@ -98,6 +98,65 @@ def effective_transformer_input(from_tensor: torch.Tensor, mask: torch.Tensor, b
     return to_tensor, valid_word_num, batch_idx, word_idx
 
 
+class EmbeddingWeights:
+    """The tables of the BERT embedding block on the device (sample/tensorflow/modeling.py:171-194):
+    word_embeddings [V,H], token_type_embeddings [Vt,H] or None, position_embeddings [P,H] or None, LayerNorm
+    gamma / beta [H]."""
+
+    def __init__(self, device, dtype: torch.dtype, word_embeddings, layernorm_gamma, layernorm_beta,
+                 token_type_embeddings=None, position_embeddings=None):
+        def up(v):
+            if v is None:
+                return None
+            if isinstance(v, np.ndarray):
+                v = torch.from_numpy(np.ascontiguousarray(v))
+            return v.to(device=device, dtype=dtype).contiguous()
+        self.word, self.type, self.pos = up(word_embeddings), up(token_type_embeddings), up(position_embeddings)
+        self.gamma, self.beta = up(layernorm_gamma), up(layernorm_beta)
+        s = _lib.EmbeddingWeights()
+        s.word_embeddings = self.word.data_ptr()
+        s.token_type_embeddings = self.type.data_ptr() if self.type is not None else None
+        s.position_embeddings = self.pos.data_ptr() if self.pos is not None else None
+        s.layernorm_gamma, s.layernorm_beta = self.gamma.data_ptr(), self.beta.data_ptr()
+        s.vocab_size = self.word.shape[0]
+        s.type_vocab_size = self.type.shape[0] if self.type is not None else 0
+        s.max_position_embeddings = self.pos.shape[0] if self.pos is not None else 0
+        self.struct = s
+        self.hidden = self.word.shape[1]
+        self.dtype = dtype
+
+
+def effective_transformer_embedding_input(input_ids: torch.Tensor, token_type_ids: Optional[torch.Tensor],
+                                          mask: torch.Tensor, embeddings: EmbeddingWeights, head_num: int,
+                                          size_per_head: int, return_host_count: bool = False):
+    """Embedding block (modeling.py:380-521) fused with EffectiveTransformerInput: packed rows straight from the ids,
+    the padded [B,S,H] embedding output is never written.  Returns what effective_transformer_input returns."""
+    lib = _lib.load()
+    _require_cuda(input_ids, mask)
+    if token_type_ids is not None:
+        _require_cuda(token_type_ids)
+    for t in (input_ids, mask) + ((token_type_ids,) if token_type_ids is not None else ()):
+        if t.dtype != torch.int32:
+            raise TypeError("ids and mask must be int32")
+    B, S = mask.shape
+    dev = mask.device
+    to_tensor = torch.empty(B, S, embeddings.hidden, dtype=embeddings.dtype, device=dev)
+    valid_word_num = torch.empty(1, dtype=torch.int32, device=dev)
+    batch_idx = torch.empty_like(mask)
+    word_idx = torch.empty_like(mask)
+    ws = _workspace(dev, "input", lib.et_input_workspace_bytes(B, S))
+    host = C.c_int32(-1)
+    h = handle(dev)
+    st = lib.et_embedding_input(h, _dtype_code(embeddings.dtype), C.byref(embeddings.struct), _p(input_ids),
+                                _p(token_type_ids), _p(mask), _p(to_tensor), _p(valid_word_num), _p(batch_idx),
+                                _p(word_idx), B, S, head_num, size_per_head, _p(ws), ws.numel(), _stream(),
+                                C.byref(host) if return_host_count else None)
+    _lib.check(st, h)
+    if return_host_count:
+        return to_tensor, valid_word_num, batch_idx, word_idx, int(host.value)
+    return to_tensor, valid_word_num, batch_idx, word_idx
+
+
 class LayerWeights:
     """The 16 tensors of one layer on the device, keyed by the attribute names of the
     reference op (tf_op/bert_transformer_op.cc:44-77)."""
@@ -226,10 +285,25 @@ class EffectiveTransformerEncoder:
         else:
             x, vwn, bidx, widx = effective_transformer_input(from_tensor, input_mask, B, S, S, hn, d)
             T = -1
-        key = tuple(from_tensor.shape)
+        return self._layers_and_output(x, vwn, bidx, widx, T, attention_mask, B, S)
+
+    def forward_ids(self, input_ids, token_type_ids, input_mask, attention_mask, embeddings: "EmbeddingWeights",
+                    sync_count: bool = True) -> torch.Tensor:
+        """Embedding block + encoder from token ids: the packed token matrix is produced directly."""
+        B, S = input_mask.shape
+        hn, d = self.head_num, self.size_per_head
+        r = effective_transformer_embedding_input(input_ids, token_type_ids, input_mask, embeddings, hn, d,
+                                                  return_host_count=sync_count)
+        x, vwn, bidx, widx = r[:4]
+        T = r[4] if sync_count else -1
+        return self._layers_and_output(x, vwn, bidx, widx, T, attention_mask, B, S)
+
+    def _layers_and_output(self, x, vwn, bidx, widx, T, attention_mask, B, S):
+        hn, d = self.head_num, self.size_per_head
+        key = tuple(x.shape)
         bufs = self._bufs.get(key)
         if bufs is None:
-            bufs = (torch.empty_like(from_tensor), torch.empty_like(from_tensor))
+            bufs = (torch.empty_like(x), torch.empty_like(x))
             self._bufs[key] = bufs
         for l, w in enumerate(self.layers):
             out = bufs[l & 1]

@@ -120,6 +120,33 @@ et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const 
                     const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor,
                     int batch_size, int seq_len, int head_num, int size_per_head, void* stream);
 
+/* ---- the step in front of the path --------------------------------------------------- */
+
+/* The tables of the BERT embedding block (sample/tensorflow/modeling.py:171-194: `word_embeddings`,
+ * `token_type_embeddings`, `position_embeddings`, then `LayerNorm/{gamma,beta}`), row-major in dtype. */
+typedef struct et_embedding_weights {
+  const void* word_embeddings;        /* [vocab_size, H]                         */
+  const void* token_type_embeddings;  /* [type_vocab_size, H] or NULL            */
+  const void* position_embeddings;    /* [max_position_embeddings, H] or NULL    */
+  const void* layernorm_gamma;        /* [H]                                     */
+  const void* layernorm_beta;         /* [H]                                     */
+  int vocab_size, type_vocab_size, max_position_embeddings;
+} et_embedding_weights;
+
+/* Embedding lookup + post-processing fused with et_input: what embedding_lookup, embedding_postprocessor
+ * (sample/tensorflow/modeling.py:380-521, dropout off) and EffectiveTransformerInputOpFunctor::Compute
+ * (tf_op/bert_transformer_op.cu.cc:266-331) do one after the other, without the padded [B,S,H] tensor in between --
+ * the reference notes that the compress belongs in front of the embedding (:295-296).
+ *   input_ids, token_type_ids (may be NULL), mask: int32 [B,S]  ->
+ *   to_tensor row t = LayerNorm(word[id] + type[type_id] + position[s]) (eps 1e-12) for the t-th valid (b,s);
+ *   valid_word_num_dev, batch_idx, word_idx exactly as et_input writes them.
+ * Ids outside their table contribute a zero row.  workspace: et_input_workspace_bytes(B, S). */
+et_status et_embedding_input(et_handle h, et_dtype dtype, const et_embedding_weights* embeddings,
+                             const int32_t* input_ids, const int32_t* token_type_ids, const int32_t* mask,
+                             void* to_tensor, int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx,
+                             int batch_size, int seq_len, int head_num, int size_per_head,
+                             void* workspace, size_t workspace_bytes, void* stream, int32_t* valid_word_num_host);
+
 /* ---- kernel-level entry points (unit tests, profiling in isolation) ----------------- */
 
 /* exclusiveScan_kernelLauncher, cuda/cuda_kernels.h:29 (cuda/cuda_kernels.cu:709-718).

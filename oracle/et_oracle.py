@@ -127,6 +127,43 @@ def input_op_fast(from_tensor, mask):
     return to_tensor, T, batch_idx, word_idx, prefix
 
 
+def embedding_postprocess(input_ids, token_type_ids, word_table, type_table, pos_table, gamma, beta, dtype: str):
+    """Padded embedding block of the reference's sample model, [B,S] ids -> [B,S,H]
+    (sample/tensorflow/modeling.py:380-521 with dropout off): output = word_table[ids];
+    output += type_table[type_ids]; output += pos_table[:S]; layer_norm (tf.contrib.layers.layer_norm: biased
+    variance + 1e-12).  Sums in the element type in that order, statistics in float.  Ids outside a table give a zero
+    row (tf.gather on a GPU).  type_table / pos_table may be None."""
+    ids = np.asarray(input_ids, dtype=np.int64)
+    B, S = ids.shape
+    H = word_table.shape[1]
+    npdt = _np_dtype(dtype)
+
+    def gather(table, idx):
+        ok = (idx >= 0) & (idx < table.shape[0])
+        rows = np.asarray(table).astype(npdt)[np.where(ok, idx, 0)]
+        return np.where(ok[..., None], rows, npdt(0)).astype(npdt)
+
+    x = gather(word_table, ids)
+    if type_table is not None:
+        t = gather(type_table, np.asarray(token_type_ids, dtype=np.int64))
+        x = hadd(x, t) if dtype == "fp16" else (x + t).astype(np.float32)
+    if pos_table is not None:
+        p = np.broadcast_to(np.asarray(pos_table).astype(npdt)[:S][None], (B, S, H))
+        x = hadd(x, p) if dtype == "fp16" else (x + p).astype(np.float32)
+    x = x.astype(np.float64)
+    mean = x.sum(axis=-1, keepdims=True) / H
+    var = ((x - mean) ** 2).sum(axis=-1, keepdims=True) / H + 1e-12
+    y = (x - mean) / np.sqrt(var) * np.asarray(gamma).astype(np.float64) + np.asarray(beta).astype(np.float64)
+    return rnd(y, dtype)
+
+
+def embedding_input(input_ids, token_type_ids, mask, word_table, type_table, pos_table, gamma, beta, dtype: str):
+    """embedding_postprocess followed by input_op (the order in which the reference runs them,
+    python/effective_transformer/__init__.py:40-45 on the output of modeling.py:171-194)."""
+    padded = embedding_postprocess(input_ids, token_type_ids, word_table, type_table, pos_table, gamma, beta, dtype)
+    return input_op_fast(padded, mask)
+
+
 def restore(from_tensor, T: int, batch_idx, word_idx, B: int, S: int):
     """EffectiveTransformerOutput: zero [B,S,H] then scatter T rows
     (tf_op/bert_transformer_op.cu.cc:351-360, cuda/cuda_kernels.cu:396-406)."""

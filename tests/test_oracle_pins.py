@@ -268,3 +268,58 @@ def test_fp16_mode_tracks_fp32_mode():
     w32 = [a.astype(np.float32) for a in w]
     got32 = o.encoder(x.astype(np.float32), mask, attr.astype(np.float32), w32, wl.heads, wl.d, "fp32")
     assert np.abs(got16.astype(np.float32) - got32).max() < 2e-2
+
+
+def test_embedding_block_against_huggingface_embeddings():
+    """The padded embedding block (word + token type + position, LayerNorm 1e-12) against transformers'
+    BertEmbeddings with the same tables; the packed form against a position-by-position loop."""
+    from transformers import BertConfig
+    from transformers.models.bert.modeling_bert import BertEmbeddings
+    rng = np.random.RandomState(11)
+    V, Vt, P, H, B, S = 97, 3, 40, 64, 4, 12
+    word = rng.randn(V, H).astype(np.float32)
+    typ = rng.randn(Vt, H).astype(np.float32)
+    pos = rng.randn(P, H).astype(np.float32)
+    gamma = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+    beta = (0.1 * rng.randn(H)).astype(np.float32)
+    ids = rng.randint(0, V, size=(B, S)).astype(np.int32)
+    tt = rng.randint(0, Vt, size=(B, S)).astype(np.int32)
+    cfg = BertConfig(vocab_size=V, hidden_size=H, max_position_embeddings=P, type_vocab_size=Vt, layer_norm_eps=1e-12,
+                     hidden_dropout_prob=0.0, num_hidden_layers=1, num_attention_heads=1, intermediate_size=4 * H,
+                     pad_token_id=0)
+    emb = BertEmbeddings(cfg).eval()
+    with torch.no_grad():
+        emb.word_embeddings.weight.copy_(torch.from_numpy(word))
+        emb.token_type_embeddings.weight.copy_(torch.from_numpy(typ))
+        emb.position_embeddings.weight.copy_(torch.from_numpy(pos))
+        emb.LayerNorm.weight.copy_(torch.from_numpy(gamma))
+        emb.LayerNorm.bias.copy_(torch.from_numpy(beta))
+        want = emb(input_ids=torch.from_numpy(ids).long(), token_type_ids=torch.from_numpy(tt).long()).numpy()
+    got = o.embedding_postprocess(ids, tt, word, typ, pos, gamma, beta, "fp32")
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+    # without the optional tables: plain LayerNorm of the word rows
+    got_w = o.embedding_postprocess(ids, None, word, None, None, gamma, beta, "fp32")
+    want_w = torch.nn.functional.layer_norm(torch.from_numpy(word[ids]), (H,), torch.from_numpy(gamma),
+                                            torch.from_numpy(beta), eps=1e-12).numpy()
+    np.testing.assert_allclose(got_w, want_w, rtol=1e-5, atol=1e-5)
+    # an id outside the vocabulary contributes a zero row
+    ids2 = ids.copy(); ids2[1, 3] = V + 5; ids2[2, 0] = -1
+    got2 = o.embedding_postprocess(ids2, tt, word, typ, pos, gamma, beta, "fp32")
+    x = typ[tt[1, 3]] + pos[3]
+    ref = (x - x.mean()) / np.sqrt(x.var() + 1e-12) * gamma + beta
+    np.testing.assert_allclose(got2[1, 3], ref, rtol=1e-5, atol=1e-5)
+    assert np.array_equal(got2[0], got[0])
+    # packed form: row t is the padded row of the t-th valid position
+    mask = (rng.rand(B, S) < 0.6).astype(np.int32)
+    packed, T, bi, wi, _ = o.embedding_input(ids, tt, mask, word, typ, pos, gamma, beta, "fp32")
+    t = 0
+    for b in range(B):
+        for s_ in range(S):
+            if mask[b, s_]:
+                assert bi[t] == b and wi[t] == s_ and np.array_equal(packed[t], got[b, s_])
+                t += 1
+    assert t == T == packed.shape[0]
+    # fp16: the sums round to half after each add
+    h = o.embedding_postprocess(ids, tt, word, typ, pos, gamma, beta, "fp16")
+    assert h.dtype == np.float16
+    np.testing.assert_allclose(h.astype(np.float32), got, rtol=2e-2, atol=2e-2)
