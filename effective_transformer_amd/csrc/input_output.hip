@@ -16,7 +16,7 @@ namespace et {
 
 namespace {
 
-constexpr int kScanThreads = 256;
+constexpr int kScanThreads = 1024;     // one element per thread and tile step; 16 wavefronts share the front sum
 constexpr int kScanWaves = kScanThreads / kWave;
 
 inline int scan_tile_for(int length) {
@@ -67,24 +67,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_index_kernel(const int32_t*
     // few tiles: add up everything in front of this tile straight from the input (it sits in L2), saving a launch
     const int n4 = blockIdx.x * tile / 4;             // int4 words in front of this tile (tile is a multiple of 4)
     const int4* in4 = reinterpret_cast<const int4*>(in);
-    int i = threadIdx.x;
-    // 32, then 8 independent loads in flight per thread: the longest front (252 KB at 64K positions) is two round
-    // trips to L2 instead of one per 4 KB
-    auto batch = [&](auto ku) {
-      constexpr int kU = decltype(ku)::value;
-      for (; i + (kU - 1) * kScanThreads < n4; i += kU * kScanThreads) {
-        int4 v[kU];
+    // 16 unpredicated loads in flight per thread (indices past the end are clamped and their values dropped): the
+    // longest front (252 KB at 64K positions) is one round trip to L2
+    constexpr int kU = 16;
+    for (int base = 0; base < n4; base += kU * kScanThreads) {
+      int4 v[kU];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) v[u] = in4[i + u * kScanThreads];
+      for (int u = 0; u < kU; ++u) v[u] = in4[min(base + u * kScanThreads + (int)threadIdx.x, n4 - 1)];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) part += v[u].x + v[u].y + v[u].z + v[u].w;
-      }
-    };
-    batch(std::integral_constant<int, 32>{});
-    batch(std::integral_constant<int, 8>{});
-    for (; i < n4; i += kScanThreads) {
-      const int4 v = in4[i];
-      part += v.x + v.y + v.z + v.w;
+      for (int u = 0; u < kU; ++u)
+        part += base + u * kScanThreads + (int)threadIdx.x < n4 ? v[u].x + v[u].y + v[u].z + v[u].w : 0;
     }
   }
   int carry = block_sum_i32(part, lds);
@@ -139,7 +131,7 @@ __global__ __launch_bounds__(256) void index_from_prefix_kernel(const int32_t* _
 }
 
 constexpr int kMoveThreads = 256;
-constexpr int kMoveUnroll = 4;
+constexpr int kMoveUnroll = 8;
 
 // Gather of packed rows: flattened over (packed row, 16-byte chunk).
 __global__ __launch_bounds__(kMoveThreads) void compress_rows_kernel(
