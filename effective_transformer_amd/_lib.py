@@ -57,6 +57,7 @@ SIGNATURES = {
                                 _vp, _sz, _vp, _ip]),
     "et_layer": (_i, [_vp, _i, C.POINTER(LayerWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                       _vp, _sz, _vp]),
+    "et_first_token": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "et_output": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "et_exclusive_scan": (_i, [_vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "et_compress": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),

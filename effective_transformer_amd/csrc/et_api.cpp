@@ -353,6 +353,22 @@ et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const 
                     head_num * size_per_head, stream);
 }
 
+et_status et_first_token(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* valid_word_num_dev,
+                         const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor, int batch_size,
+                         int seq_len, int hidden_dim, void* stream) {
+  et_status s = enter(h);
+  if (s != ET_OK) return s;
+  Scope scope(h);
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
+  ET_REQUIRE(h, from_tensor && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  const size_t row_bytes = (size_t)hidden_dim * et::elem_size(to_dt(dtype));
+  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
+  et::launch_first_token(to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size * seq_len,
+                         batch_size, (int)row_bytes, (hipStream_t)stream);
+  return check_launch(h, "first token gather");
+}
+
 et_status et_exclusive_scan(et_handle h, int32_t* d_out, const int32_t* d_in, int length, void* workspace,
                             size_t workspace_bytes, void* stream) {
   et_status s = enter(h);

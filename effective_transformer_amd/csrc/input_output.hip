@@ -253,7 +253,39 @@ __global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restric
   for (int b = prev + 1; b <= last; ++b) seq_start[b] = t;
 }
 
+// to[b,:] = row of the packed matrix that sits at position 0 of sequence b, zeros where sequence b has no token
+// there.  One wavefront per packed row (plus one past the end): the row that opens a sequence serves that sequence
+// and zeroes the token-less sequences in front of it, like seq_start_kernel walks the batch.
+__global__ __launch_bounds__(256) void first_token_kernel(u32x4* __restrict__ to, const u32x4* __restrict__ from,
+                                                          const int32_t* __restrict__ batch_idx,
+                                                          const int32_t* __restrict__ word_idx,
+                                                          const int32_t* __restrict__ rows_dev, int rows_bound,
+                                                          int batch, int cpr) {
+  const int T = rows_dev ? min(*rows_dev, rows_bound) : rows_bound;
+  const int t = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (t > T) return;
+  const int prev = t == 0 ? -1 : min(batch_idx[t - 1], batch - 1);
+  const int cur = t == T ? batch : min(batch_idx[t], batch - 1);
+  if (cur == prev) return;                          // not the first row of its sequence
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (int b = prev + 1; b < min(cur, batch); ++b)
+    for (int c = lane; c < cpr; c += kWave) to[(size_t)b * cpr + c] = zero;
+  if (t < T) {
+    const bool at0 = word_idx[t] == 0;
+    for (int c = lane; c < cpr; c += kWave) to[(size_t)cur * cpr + c] = at0 ? from[(size_t)t * cpr + c] : zero;
+  }
+}
+
 }  // namespace
+
+void launch_first_token(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
+                        const int32_t* rows_dev, int rows_bound, int batch, int row_bytes, hipStream_t stream) {
+  const int n = rows_bound + 1;
+  const int per_wg = 256 / kWave;
+  first_token_kernel<<<(n + per_wg - 1) / per_wg, 256, 0, stream>>>((u32x4*)to, (const u32x4*)from, batch_idx, word_idx,
+                                                                    rows_dev, rows_bound, batch, row_bytes / 16);
+}
 
 size_t scan_scratch_words(int length) {
   const int tile = scan_tile_for(length);

@@ -31,6 +31,9 @@ void launch_compress_rows(const void* from, void* to, const int32_t* batch_idx, 
 // to[B*S rows] = 0 at padding, from[t] at batch_idx[t]*S + word_idx[t]; indices ascending.
 void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
                          const int32_t* rows_dev, int batch, int seq_len, int row_bytes, hipStream_t stream);
+// to[b,:] = packed row at position 0 of sequence b (zeros if there is none); indices ascending.
+void launch_first_token(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
+                        const int32_t* rows_dev, int rows_bound, int batch, int row_bytes, hipStream_t stream);
 // seq_start[b] = first packed row of sequence b, b in [0,B]; seq_start[B] = T.
 void launch_seq_start(const int32_t* batch_idx, const int32_t* rows_dev, int rows_bound, int batch,
                       int32_t* seq_start, hipStream_t stream);

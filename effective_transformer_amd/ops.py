@@ -247,6 +247,22 @@ def effective_transformer_output(from_tensor: torch.Tensor, valid_word_num: torc
     return to_tensor
 
 
+def effective_transformer_first_token(from_tensor: torch.Tensor, valid_word_num: torch.Tensor, batch_idx: torch.Tensor,
+                                      word_idx: torch.Tensor) -> torch.Tensor:
+    """[B,H]: the row at position 0 of every sequence, read from the packed matrix (what the pooler takes from
+    `sequence_output[:, 0]`, sample/tensorflow/modeling.py:224-232); zeros where position 0 holds no token."""
+    lib = _lib.load()
+    _require_cuda(from_tensor, valid_word_num, batch_idx, word_idx)
+    B, S = batch_idx.shape
+    H = from_tensor.shape[-1]
+    out = torch.empty(B, H, dtype=from_tensor.dtype, device=from_tensor.device)
+    h = handle(from_tensor.device)
+    st = lib.et_first_token(h, _dtype_code(from_tensor.dtype), _p(from_tensor), _p(valid_word_num), _p(batch_idx),
+                            _p(word_idx), _p(out), B, S, H, _stream())
+    _lib.check(st, h)
+    return out
+
+
 # --------------------------------------------------------------------------- the glue
 
 class EffectiveTransformerEncoder:

@@ -147,6 +147,15 @@ et_status et_embedding_input(et_handle h, et_dtype dtype, const et_embedding_wei
                              int batch_size, int seq_len, int head_num, int size_per_head,
                              void* workspace, size_t workspace_bytes, void* stream, int32_t* valid_word_num_host);
 
+/* The consumer side of the same fusion: the first token of every sequence straight from the packed matrix, i.e.
+ * what `sequence_output[:, 0:1, :]` (the pooler's input, sample/tensorflow/modeling.py:224-232) reads after
+ * EffectiveTransformerOutput, without materialising the padded [B,S,H] tensor.
+ *   from_tensor [T,H] packed, batch_idx / word_idx as written by et_input  ->  to_tensor [B,H]
+ * (zeros for a sequence whose position 0 holds no token). */
+et_status et_first_token(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* valid_word_num_dev,
+                         const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor,
+                         int batch_size, int seq_len, int hidden_dim, void* stream);
+
 /* ---- kernel-level entry points (unit tests, profiling in isolation) ----------------- */
 
 /* exclusiveScan_kernelLauncher, cuda/cuda_kernels.h:29 (cuda/cuda_kernels.cu:709-718).

@@ -119,3 +119,27 @@ def test_encoder_from_ids_matches_encoder_on_padded_embeddings():
     torch.cuda.synchronize()
     # the fused path rounds like the oracle up to the LayerNorm's last ulp; after two layers the outputs agree closely
     np.testing.assert_allclose(got.float().cpu().numpy(), want.float().cpu().numpy(), rtol=0, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("case", ["prefix", "holes", "empty_sequences", "all_empty"])
+def test_first_token_equals_restore_then_slice(dtype, case):
+    from effective_transformer_amd import ops
+    print("first_token", dtype, case, flush=True)
+    rng = np.random.RandomState(17)
+    B, S, H = 37, 24, 128
+    x = o.rnd(rng.randn(B, S, H), dtype)
+    if case == "prefix":
+        mask = (np.arange(S)[None, :] < rng.randint(1, S + 1, size=B)[:, None]).astype(np.int32)
+    elif case == "holes":
+        mask = (rng.rand(B, S) < 0.5).astype(np.int32)
+    elif case == "empty_sequences":
+        mask = (np.arange(S)[None, :] < rng.randint(1, S + 1, size=B)[:, None]).astype(np.int32)
+        mask[[0, 5, 6, 7, B - 1]] = 0
+    else:
+        mask = np.zeros((B, S), np.int32)
+    to, vwn, bi, wi = ops.effective_transformer_input(dev(x), dev(mask), B, S, S, H // 64, 64)
+    got = ops.effective_transformer_first_token(to, vwn, bi, wi).cpu().numpy()
+    packed, T, obi, owi, _ = o.input_op_fast(x, mask)
+    want = o.restore(packed, T, obi, owi, B, S)[:, 0, :]
+    assert np.array_equal(got, want)
