@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void transpose_rm_padding_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// fused attention, size_per_head = 64, seq_len <= 128.
+// fused attention, size_per_head = 64, seq_len <= 128 (longer sequences: attention_long_kernel below).
 //
 // One workgroup (4 wavefronts) per (sequence, group of up to 4 heads).  What does not depend on the
 // head is done once: token positions, the zero fill of key/value slots without a token (so that a
@@ -525,11 +525,316 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
                                                    hpw, scaler);
 }
 
+
+// ------------------------------------------------------------------------------------------
+// fused attention for 128 < seq_len <= 512: one workgroup (4 wavefronts) per (64 queries, head, sequence).
+// The scores of a wavefront's 16 queries against all keys stay in registers (4 per lane and 16-key tile); K and
+// V pass through LDS in chunks of 128 keys (K chunks first, the softmax over the registers, then V chunks), so the
+// LDS footprint does not grow with the sequence.  Q comes straight from global memory: the MFMA operand of a lane
+// is 16 (fp16) or 64 (fp32) contiguous bytes of its query's row.  Arithmetic and rounding points are those of
+// the kernel above; key tiles beyond the last token skip their MFMAs (score 0, value 0).
+// ------------------------------------------------------------------------------------------
+constexpr int kLongChunkTiles = 8;                 // 128 keys per LDS chunk
+constexpr int kLongChunk = kLongChunkTiles * 16;
+
+template <typename T>
+struct LongSmem {
+  static constexpr int kQS = AttnCfg<T>::kQkStride;
+  static constexpr int kVR = kD + 16;                                  // fp16 V rows
+  static constexpr int kVS = kLongChunk + AttnCfg<T>::kVtPad;          // fp32 V^T rows
+  static constexpr size_t kKBytes = (size_t)kLongChunk * kQS * sizeof(T);
+  static constexpr size_t kVBytes = sizeof(T) == 2 ? (size_t)kLongChunk * kVR * sizeof(T) : (size_t)kD * kVS * sizeof(T);
+  static constexpr size_t kTileBytes = kKBytes > kVBytes ? kKBytes : kVBytes;   // K and V chunks take turns
+};
+
+template <typename T, int NKT>
+__global__ __launch_bounds__(kAttnThreads) void attention_long_kernel(
+    const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
+    const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ word_idx, int seq_len, int heads, float scaler) {
+  using Sm = LongSmem<T>;
+  using C = Chunk16<T>;
+  using V16 = typename C::vec;
+  constexpr int kQS = Sm::kQS, kVR = Sm::kVR, kVS = Sm::kVS;
+  constexpr int kSp = NKT * 16;
+  constexpr int kCpr = kD / C::kElems;
+  constexpr int kChunks = NKT / kLongChunkTiles;
+  constexpr int CPT = kLongChunk * kCpr / kAttnThreads;      // 16-byte pieces of a chunk per thread
+  typedef T mask4 __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* Ks = reinterpret_cast<T*>(smem_raw);                    // K chunk, later V chunk
+  T* Vs = Ks;
+  int* tok_of_pos = reinterpret_cast<int*>(smem_raw + Sm::kTileBytes);
+
+  const int b = blockIdx.z, head = blockIdx.y, qblock = blockIdx.x;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  const int len = t1 - t0;
+  if (len <= 0) return;
+  const int H = heads * kD;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int l16 = lane & 15, g = lane >> 4;
+
+  const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
+  const int n_tiles = last_pos / 16 + 1;                     // 16-row tiles that hold at least one token
+  if (qblock * 4 >= n_tiles) return;                         // no token among this workgroup's queries
+  for (int i = threadIdx.x; i < kSp; i += kAttnThreads) tok_of_pos[i] = -1;
+  __syncthreads();
+  for (int tt = threadIdx.x; tt < len; tt += kAttnThreads) {
+    const int pos = word_idx[t0 + tt];
+    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = t0 + tt;
+  }
+  __syncthreads();
+
+  // element offset of (token t / position pos, this head) in the source matrices
+  auto src_off = [&](int t, int pos) -> size_t {
+    return layout == 1 ? (size_t)t * packed_ld + head * kD : (((size_t)b * heads + head) * seq_len + pos) * kD;
+  };
+  // stage rows [c0, c0 + 128) of `src` row-major (stride `stride` elements) into LDS, zeros where no token sits
+  auto stage_rows = [&](const T* __restrict__ src, T* lds, int stride, int c0) {
+    V16 r[CPT];
+    int tk[CPT];
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+      const int i = threadIdx.x + k * kAttnThreads;
+      const int row = i / kCpr, c = i - row * kCpr;
+      const int pos = c0 + row;
+      tk[k] = pos < kSp ? tok_of_pos[pos] : -1;
+#pragma unroll
+      for (int j = 0; j < C::kElems; ++j) r[k][j] = (T)0;
+      if (tk[k] >= 0) r[k] = *reinterpret_cast<const V16*>(src + src_off(tk[k], pos) + c * C::kElems);
+    }
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+      const int i = threadIdx.x + k * kAttnThreads;
+      const int row = i / kCpr, c = i - row * kCpr;
+      *reinterpret_cast<V16*>(lds + row * stride + c * C::kElems) = r[k];
+    }
+  };
+
+  const int qt = qblock * 4 + wave;                          // this wavefront's 16-query tile
+  const bool active = qt < n_tiles;                          // wave-uniform
+  const int q = qt * 16 + l16;
+  const int tq = (active && q < kSp) ? tok_of_pos[q] : -1;
+  const T* mrow = attr_mask + ((size_t)b * seq_len + min(q, seq_len - 1)) * seq_len;
+  const bool vec_mask = (seq_len & 3) == 0;
+
+  // Q operand of this lane (zeros for a query position without a token: its result is never stored)
+  half8 bqh[2];
+  float bqf[16];
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bqh[ks][j] = (_Float16)0;
+      if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + src_off(tq, q) + ks * 32 + g * 8);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float4v v4 = {0.f, 0.f, 0.f, 0.f};
+      if (tq >= 0) v4 = *reinterpret_cast<const float4v*>(q_src + src_off(tq, q) + g * 16 + i * 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bqf[i * 4 + j] = v4[j];
+    }
+  }
+
+  // ---- S^T = K Q^T chunk by chunk, bias added on the way ------------------------------------------
+  float s[NKT][4];
+#pragma unroll
+  for (int ch = 0; ch < kChunks; ++ch) {
+    const bool chunk_has_tokens = ch * kLongChunkTiles < n_tiles;       // workgroup-uniform
+    if (chunk_has_tokens) {
+      __syncthreads();                                                  // previous chunk fully consumed
+      stage_rows(k_src, Ks, kQS, ch * kLongChunk);
+      __syncthreads();
+    }
+    if (active) {
+#pragma unroll
+      for (int kc = 0; kc < kLongChunkTiles; ++kc) {
+        const int kt = ch * kLongChunkTiles + kc;
+        float4v acc = {0.f, 0.f, 0.f, 0.f};
+        if (kt < n_tiles) {
+          if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+              const half8 a = *reinterpret_cast<const half8*>(Ks + (kc * 16 + l16) * kQS + ks * 32 + g * 8);
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bqh[ks], acc, 0, 0, 0);
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kc * 16 + l16) * kQS + g * 16 + i * 4);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bqf[i * 4 + j], acc, 0, 0, 0);
+            }
+          }
+        }
+        const int key0 = kt * 16 + g * 4;
+        mask4 m4 = {(T)0, (T)0, (T)0, (T)0};
+        if (vec_mask) {
+          if (key0 < seq_len) m4 = *reinterpret_cast<const mask4*>(mrow + key0);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (key0 + r < seq_len) m4[r] = mrow[key0 + r];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float sc = sizeof(T) == 2 ? h2f(f2h(acc[r])) : acc[r];      // the score is stored in the element type
+          s[kt][r] = key0 + r < seq_len ? sc * scaler + (1.0f - (float)m4[r]) * -10000.0f : -INFINITY;
+        }
+      }
+    }
+  }
+
+  // ---- masked softmax over the registers ---------------------------------------------------------------
+  if (active) {
+    float mx = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][r]);
+    mx = xor_lanes_16_32_max(mx) * kLog2e;
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[kt][r] = __builtin_amdgcn_exp2f(s[kt][r] * kLog2e - mx);
+        sum += s[kt][r];
+      }
+    sum = xor_lanes_16_32_sum(sum) + 1e-6f;
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
+  }
+
+  // ---- O^T = V^T P^T chunk by chunk ----------------------------------------------------------------------
+  float4v o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ch = 0; ch < kChunks; ++ch) {
+    if (ch * kLongChunkTiles >= n_tiles) break;                         // workgroup-uniform: no token, value 0
+    __syncthreads();
+    if constexpr (sizeof(T) == 2) {
+      stage_rows(v_src, Vs, kVR, ch * kLongChunk);
+    } else {
+      // fp32 keeps V^T: feature rows, key columns
+#pragma unroll
+      for (int k = 0; k < CPT; ++k) {
+        const int i = threadIdx.x + k * kAttnThreads;
+        const int row = i / kCpr, c = i - row * kCpr;
+        const int pos = ch * kLongChunk + row;
+        const int tk = pos < kSp ? tok_of_pos[pos] : -1;
+        V16 r = {0.f, 0.f, 0.f, 0.f};
+        if (tk >= 0) r = *reinterpret_cast<const V16*>(v_src + src_off(tk, pos) + c * C::kElems);
+#pragma unroll
+        for (int j = 0; j < C::kElems; ++j) Vs[(c * C::kElems + j) * kVS + row] = r[j];
+      }
+    }
+    __syncthreads();
+    if (!active) continue;
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int kp = 0; kp < kLongChunkTiles / 2; ++kp) {
+        const int kt = ch * kLongChunkTiles + 2 * kp;
+        if (kt < n_tiles) {
+          half8 p;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            p[r] = f2h(s[kt][r]);
+            p[4 + r] = f2h(s[kt + 1][r]);
+          }
+          typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+          typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+          u2 raw[8];
+#pragma unroll
+          for (int kk = 0; kk < 8; ++kk) {
+            const int key = kp * 32 + (kk >> 2) * 16 + g * 4 + (kk & 3);
+            raw[kk] = *reinterpret_cast<const u2*>(Vs + key * kVR + l16 * 4);
+          }
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            u4 lo, hi;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+              lo[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x05040100u);
+              hi[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x07060302u);
+            }
+            o[2 * jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, lo), p, o[2 * jj], 0, 0, 0);
+            o[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, hi), p, o[2 * jj + 1], 0, 0, 0);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int kc = 0; kc < kLongChunkTiles; ++kc) {
+        const int kt = ch * kLongChunkTiles + kc;
+        if (kt < n_tiles) {
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) {
+            const float4v a4 = *reinterpret_cast<const float4v*>(Vs + (dt * 16 + l16) * kVS + kc * 16 + g * 4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[kt][r], o[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  if (tq >= 0) {
+    if constexpr (sizeof(T) == 2) {
+      half8 v0, v1;
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v0[4 * r + j] = f2h(o[j][r]);
+          v1[4 * r + j] = f2h(o[j][2 + r]);
+        }
+      T* orow = dst + (size_t)tq * H + head * kD + g * 16;
+      *reinterpret_cast<half8*>(orow) = v0;
+      *reinterpret_cast<half8*>(orow + 8) = v1;
+    } else {
+      T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        float4v v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = o[dt][r];
+        *reinterpret_cast<float4v*>(orow + dt * 16) = v;
+      }
+    }
+  }
+}
+
+template <typename T, int NKT>
+void attention_long_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
+                           void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
+                           float scaler, hipStream_t stream) {
+  const size_t smem = LongSmem<T>::kTileBytes + (size_t)NKT * 16 * sizeof(int);
+  auto kern = attention_long_kernel<T, NKT>;
+  dim3 grid(NKT / 4, heads, batch);
+  kern<<<grid, kAttnThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld, (const T*)attr_mask,
+                                             (T*)dst, seq_start, word_idx, seq_len, heads, scaler);
+}
+
 template <typename T>
 void attention_dispatch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                         void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                         float scaler, hipStream_t stream) {
-  if (seq_len <= 32)
+  if (seq_len > 256)
+    attention_long_launch<T, 32>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                                 scaler, stream);
+  else if (seq_len > 128)
+    attention_long_launch<T, 16>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                                 scaler, stream);
+  else if (seq_len <= 32)
     attention_launch<T, 2>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
                            scaler, stream);
   else if (seq_len <= 64)
@@ -588,7 +893,7 @@ void launch_transpose_rm_padding(DType t, const void* src, void* dst, const int3
 
 bool attention_supported(DType t, int seq_len, int d) {
   (void)t;
-  return d == kD && seq_len >= 1 && seq_len <= 128;
+  return d == kD && seq_len >= 1 && seq_len <= 512;
 }
 
 void launch_attention(DType t, const void* q, const void* k, const void* v, int layout, int packed_ld,

@@ -263,7 +263,7 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   if (workspace_bytes < ws.total) return fail(h, ET_WORKSPACE_TOO_SMALL, "et_layer needs et_layer_workspace_bytes(...)");
   const et::DType dt = to_dt(dtype);
   if (!et::attention_supported(dt, S, size_per_head))
-    return fail(h, ET_UNSUPPORTED, "attention kernel supports size_per_head == 64 and seq_len <= 128");
+    return fail(h, ET_UNSUPPORTED, "attention kernels support size_per_head == 64 and seq_len <= 512");
   if (!et::gemm_supported(dt, H, H, 3) || !et::gemm_supported(dt, F, H, 1) || !et::gemm_supported(dt, H, F, 1))
     return fail(h, ET_UNSUPPORTED, "hidden size not supported by the GEMM kernels");
   if ((uint64_t)B * S * F * et::elem_size(dt) > 0xffffffffull)
@@ -521,7 +521,7 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
   if (workspace_bytes < et_seq_workspace_bytes(batch_size))
     return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
   if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
-    return fail(h, ET_UNSUPPORTED, "attention kernel supports size_per_head == 64 and seq_len <= 128");
+    return fail(h, ET_UNSUPPORTED, "attention kernels support size_per_head == 64 and seq_len <= 512");
   if (qkv_layout == 1 && ((size_t)packed_ld * et::elem_size(to_dt(dtype))) % 16 != 0)
     return fail(h, ET_UNSUPPORTED, "packed_ld bytes must be a multiple of 16");
   hipStream_t st = (hipStream_t)stream;

@@ -167,3 +167,19 @@ def test_error_paths():
     with pytest.raises(TypeError):
         ops.effective_transformer_input(x.to(torch.bfloat16), mask, wl.B, wl.S, wl.S, wl.heads, wl.d)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_long_sequences_layer_against_oracle(dtype):
+    """seq_len 256 (beyond the 128 positions the resident-K/V attention kernel holds): two layers against the oracle."""
+    print("encoder S=256", dtype, flush=True)
+    wl = o.Workload("long", 77, dtype, 2, 6, 256, 4, 64, 1024, 40, 257)
+    rng = np.random.RandomState(wl.seed)
+    lens, mask, attr = o.make_masks(wl, rng)
+    x = o.rnd(rng.randn(wl.B, wl.S, wl.H), dtype)
+    weights = []
+    for _ in range(2):
+        weights.extend(o.make_layer_weights(wl, rng, True))
+    w = dict(wl=wl, lens=lens, mask=mask, attr_mask=attr, x=x, weights=weights)
+    got = run_encoder(w)
+    _check(got, _oracle(w), mask, dtype)

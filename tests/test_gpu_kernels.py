@@ -240,7 +240,10 @@ def test_softmax(k, dtype, S):
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 @pytest.mark.parametrize("S,holes,weird", [(5, False, False), (32, False, False), (64, False, False),
-                                           (64, True, True), (100, True, False), (128, False, True), (21, True, True)])
+                                           (64, True, True), (100, True, False), (128, False, True), (21, True, True),
+                                           # beyond 128 positions: the chunked kernel (K and V in 128-key chunks)
+                                           (129, False, False), (200, True, True), (256, False, False),
+                                           (300, True, False), (384, False, True), (512, False, False), (509, True, True)])
 def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
     print("attention", dtype, S, holes, weird, flush=True)
     p = _attn_problem(S + 1, 5, S, 2, dtype, holes=holes, weird_mask=weird)
