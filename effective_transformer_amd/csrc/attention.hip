@@ -510,12 +510,7 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
   constexpr int CPT = (NKT * 16 * kCpr + kAttnThreads - 1) / kAttnThreads;
   constexpr bool PF = CPT <= 4;                // more than 4 chunks x 3 matrices in flight would not fit the registers
   auto kern = attention_kernel<T, NKT, CPT, PF>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)Sm::kBytes);
-    attr_set = true;
-  }
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Sm::kBytes);
   // a workgroup serves up to 4 heads of one sequence: mask rows, positions and zero fill are shared by them
   int hpw = 4;
   while (hpw > 1 && (long)batch * ((heads + hpw - 1) / hpw) < 2048) hpw >>= 1;   // small batches: more workgroups

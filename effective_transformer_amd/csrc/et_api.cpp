@@ -11,8 +11,26 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "kernels.hpp"
+
+namespace et {
+
+void allow_dynamic_lds(const void* kernel, int bytes) {
+  static std::mutex mu;
+  static std::vector<std::pair<const void*, int>> done;      // (kernel, device) pairs already raised
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+  std::lock_guard<std::mutex> lock(mu);
+  for (const auto& e : done)
+    if (e.first == kernel && e.second == dev) return;
+  (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (dev >= 0) done.emplace_back(kernel, dev);
+}
+
+}  // namespace et
 
 struct et_context {
   int device = 0;

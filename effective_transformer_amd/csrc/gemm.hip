@@ -614,12 +614,7 @@ template <int MI>
 void launch_f16(GemmArgs a, hipStream_t stream) {
   using Tile = HTile<MI>;
   auto kern = gemm_f16_kernel<MI>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)Tile::SMEM_BYTES);
-    attr_set = true;
-  }
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Tile::SMEM_BYTES);
   a.tiles_m = (a.m_bound + Tile::BM - 1) / Tile::BM;
   a.tiles_n = (a.n + kHBN - 1) / kHBN;
   const int total = a.tiles_m * a.tiles_n * a.groups;
@@ -628,24 +623,20 @@ void launch_f16(GemmArgs a, hipStream_t stream) {
 }
 
 int device_cu_count() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
+  constexpr int kMaxDevices = 64;
+  static int cus[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  if (cus[dev] == 0) {
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
-    if (cus <= 0) cus = 256;
+    cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
-  return cus;
+  return cus[dev];
 }
 
 template <bool BT>
 void launch_f16_persistent(GemmArgs a, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_f16_persistent_kernel<BT>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kPSmem);
-    attr_set = true;
-  }
+  allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel<BT>), kPSmem);
   a.tiles_m = (a.m_bound + kPBM - 1) / kPBM;
   a.tiles_n = (a.n + kPBN - 1) / kPBN;
   const int total = a.tiles_m * a.tiles_n * a.groups;

@@ -12,6 +12,10 @@ namespace et {
 enum class DType : int { F32 = 0, F16 = 1 };
 inline size_t elem_size(DType t) { return t == DType::F32 ? 4 : 2; }
 
+// Kernels that need more than 64 KB of dynamic LDS raise the limit once per (kernel, device): the attribute belongs
+// to the device a module is loaded on, and a process may hold handles on several GPUs.  (et_api.cpp)
+void allow_dynamic_lds(const void* kernel, int bytes);
+
 // ---- input_output.hip --------------------------------------------------------------------
 // Number of int32 words of scratch the scan needs for `length` elements.
 size_t scan_scratch_words(int length);
