@@ -200,12 +200,12 @@ def main():
     import numpy as np
     import torch
     from effective_transformer_amd import _lib, ops
-    from oracle import et_oracle as o
+    from effective_transformer_amd.sample import workloads
 
     _lib.load()
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
-    w = o.make_workload(a.workload)
+    w = workloads.make_workload(a.workload)
     wl = w["wl"]
     dt = torch.float16 if wl.dtype == "fp16" else torch.float32
     enc = ops.EffectiveTransformerEncoder(wl.layers, wl.heads, wl.d, w["weights"], dt, "cuda:0")

@@ -41,6 +41,9 @@ def handle(device: torch.device) -> C.c_void_p:
 
 
 def _workspace(device: torch.device, kind: str, nbytes: int) -> torch.Tensor:
+    """One scratch buffer per (GPU, kind), grown on demand and shared by every call of this module: calls that
+    overlap on different streams of one GPU would race on it (the C ABI itself takes the workspace from the
+    caller, so such callers pass their own)."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), kind)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
