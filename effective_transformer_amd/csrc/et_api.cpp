@@ -300,7 +300,6 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   void* inter = base + ws.inter;
   int32_t* seq_start = (int32_t*)(base + ws.seq);
 
-  et::launch_seq_start(batch_idx, T, rows, B, seq_start, st);
   // The large-M fp16 GEMM reads k-contiguous weights with fewer LDS instructions; for the wide projections that is
   // worth a transposed copy in the workspace per call (the caller's weights stay as they are).
   const bool t_qkv = et::gemm_prefers_transposed_b(dt, rows, 3 * H, H, H, 3);
@@ -321,7 +320,9 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
     if (t_o) jobs.add(w->attr_output_kernel, wt_o, H, H);
     if (t_up) jobs.add(w->inter_kernel, wt_up, H, F);
     if (t_down) jobs.add(w->output_kernel, wt_down, F, H);
-    et::launch_transpose_weights(jobs, st);
+    // one launch builds the sequence start table and the transposed copies
+    const et::SeqStartJob seq{batch_idx, T, rows, B, seq_start};
+    et::launch_transpose_weights(jobs, st, &seq);
   }
   // Q = from.Wq + bq, K = to.Wk + bk, V = to.Wv + bv into one [T,3H] buffer (bert_transformer_op.cu.cc:105-156)
   et::GemmGroups g3;

@@ -115,4 +115,15 @@ __device__ __forceinline__ uint32_t div_by(uint32_t n, const fastdiv& f) {
 __device__ __forceinline__ float h2f(_Float16 h) { return (float)h; }
 __device__ __forceinline__ _Float16 f2h(float f) { return (_Float16)f; }   // v_cvt_f16_f32, round-to-nearest-even
 
+// seq_start[b] = first packed row of sequence b (b in [0, batch]; seq_start[batch] = T), written by the thread that
+// owns packed row t in [0, T]: it covers the sequences that begin at t (token-less sequences included).
+__device__ __forceinline__ void seq_start_for_row(const int32_t* __restrict__ batch_idx, int T, int t, int batch,
+                                                  int32_t* __restrict__ seq_start) {
+  if (t > T) return;
+  const int prev = t == 0 ? -1 : batch_idx[t - 1];
+  const int cur = t == T ? batch : min(batch_idx[t], batch - 1);
+  const int last = t == T ? batch : cur;         // entries (prev, last] start at t
+  for (int b = prev + 1; b <= last; ++b) seq_start[b] = t;
+}
+
 }  // namespace et

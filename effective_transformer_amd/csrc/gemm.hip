@@ -662,12 +662,19 @@ bool use_persistent(int m_bound, int ldc, int n, int k, int groups) {
 struct TransposeArgs {
   TransposeJobs jobs;
   int tile_begin[TransposeJobs::kMax + 1];
+  SeqStartJob seq;             // blocks from tile_begin[kMax] on build the sequence start table (seq_start != null)
 };
 constexpr int kTrTile = 64;
 constexpr int kTrStride = kTrTile + 8;    // halves; 144-byte rows keep the 16-byte row reads aligned
 
 __global__ __launch_bounds__(256) void transpose_weights_kernel(TransposeArgs args) {
   __shared__ __attribute__((aligned(16))) _Float16 tile[kTrTile * kTrStride];
+  if ((int)blockIdx.x >= args.tile_begin[TransposeJobs::kMax]) {
+    const int T = args.seq.rows_dev ? min(*args.seq.rows_dev, args.seq.rows_bound) : args.seq.rows_bound;
+    seq_start_for_row(args.seq.batch_idx, T, ((int)blockIdx.x - args.tile_begin[TransposeJobs::kMax]) * 256 + threadIdx.x,
+                      args.seq.batch, args.seq.seq_start);
+    return;
+  }
   int job = 0;
   while (job + 1 < args.jobs.count && (int)blockIdx.x >= args.tile_begin[job + 1]) ++job;
   const int K = args.jobs.k[job], N = args.jobs.n[job];
@@ -709,8 +716,8 @@ bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int 
   return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && (long)n * groups >= 2L * k;
 }
 
-void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream) {
-  if (jobs.count == 0) return;
+void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, const SeqStartJob* seq) {
+  if (jobs.count == 0 && seq == nullptr) return;
   TransposeArgs a;
   a.jobs = jobs;
   int total = 0;
@@ -719,6 +726,8 @@ void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream) {
     total += ((jobs.k[j] + kTrTile - 1) / kTrTile) * ((jobs.n[j] + kTrTile - 1) / kTrTile);
   }
   for (int j = jobs.count; j <= TransposeJobs::kMax; ++j) a.tile_begin[j] = total;
+  a.seq = seq ? *seq : SeqStartJob{nullptr, nullptr, 0, 0, nullptr};
+  if (seq) total += (seq->rows_bound + 1 + 255) / 256;
   transpose_weights_kernel<<<total, 256, 0, stream>>>(a);
 }
 

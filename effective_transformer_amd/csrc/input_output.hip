@@ -245,12 +245,7 @@ __global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restric
                                                         const int32_t* __restrict__ rows_dev, int rows_bound,
                                                         int batch, int32_t* __restrict__ seq_start) {
   const int T = rows_dev ? min(*rows_dev, rows_bound) : rows_bound;
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t > T) return;
-  const int prev = t == 0 ? -1 : batch_idx[t - 1];
-  const int cur = t == T ? batch : min(batch_idx[t], batch - 1);
-  const int last = t == T ? batch : cur;         // entries (prev, last] start at t
-  for (int b = prev + 1; b <= last; ++b) seq_start[b] = t;
+  seq_start_for_row(batch_idx, T, blockIdx.x * 256 + threadIdx.x, batch, seq_start);
 }
 
 // to[b,:] = row of the packed matrix that sits at position 0 of sequence b, zeros where sequence b has no token

@@ -103,7 +103,15 @@ struct TransposeJobs {
   int count = 0;
   void add(const void* s, void* d, int k_, int n_) { src[count] = s; dst[count] = d; k[count] = k_; n[count] = n_; ++count; }
 };
-void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream);
+// The layer needs the per-sequence start table as well; `seq` (optional) makes the same launch build it, which saves a
+// launch per layer.
+struct SeqStartJob {
+  const int32_t* batch_idx;
+  const int32_t* rows_dev;
+  int rows_bound, batch;
+  int32_t* seq_start;
+};
+void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, const SeqStartJob* seq = nullptr);
 void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k,
                  const int32_t* rows_dev, hipStream_t stream);
 
