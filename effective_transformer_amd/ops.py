@@ -16,7 +16,7 @@ import torch
 from . import _lib
 
 _handles: Dict[int, C.c_void_p] = {}
-_workspaces: Dict[Tuple[int, str], torch.Tensor] = {}
+_workspaces: Dict[Tuple[int, int, str], torch.Tensor] = {}
 _lock = threading.Lock()
 
 
@@ -41,10 +41,10 @@ def handle(device: torch.device) -> C.c_void_p:
 
 
 def _workspace(device: torch.device, kind: str, nbytes: int) -> torch.Tensor:
-    """One scratch buffer per (GPU, kind), grown on demand and shared by every call of this module: calls that
-    overlap on different streams of one GPU would race on it (the C ABI itself takes the workspace from the
-    caller, so such callers pass their own)."""
-    key = (device.index if device.index is not None else torch.cuda.current_device(), kind)
+    """One scratch buffer per (GPU, stream, kind), grown on demand: calls queued on one stream run in order and may
+    share it, calls on different streams get their own."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    key = (idx, torch.cuda.current_stream(idx).cuda_stream, kind)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
