@@ -758,7 +758,11 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
       if (g.b_transposed) launch_f16_persistent<true>(a, stream);
       else launch_f16_persistent<false>(a, stream);
     } else {
-      launch_f16<4>(a, stream);                             // few tiles: 128-row tiles spread over more CUs
+      // less than a round of tiles: the time is the latency of one tile's k loop, which is shorter for 64-row tiles
+      // (two of their workgroups fit a CU); from about two tiles per CU on the 128-row tile is the better one
+      const long small = (long)((m_bound + 63) / 64) * ((n + kHBN - 1) / kHBN) * g.groups;
+      if (small <= 2L * device_cu_count()) launch_f16<2>(a, stream);
+      else launch_f16<4>(a, stream);
     }
   } else {
     a.tiles_m = (m_bound + kFBM - 1) / kFBM;
