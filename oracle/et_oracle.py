@@ -23,6 +23,8 @@ tests/test_oracle_pins.py):
   add_bias_input_layernorm ... pinned against torch layer_norm(eps=1e-6).
   softmax ... pinned against torch.softmax with the additive -10000 mask.
   add_qkv_bias_padding / transpose_rm_padding ... pinned by round trip + brute force.
+  embedding_postprocess / embedding_input ... pinned against transformers' BertEmbeddings with the
+      same tables, torch layer_norm(eps=1e-12) and a position-by-position loop.
   layer / encoder ... pinned against a HuggingFace BertLayer built from a local
       config and against tf_graph_encoder (the reference benchmark's own check).
   cuBLAS half-accumulate ordering and device-intrinsic ULP behaviour (__expf,
