@@ -183,7 +183,8 @@ struct AttnSmem {
   static constexpr int kSp = NKT * 16;
   static constexpr int kVtStride = kSp + AttnCfg<T>::kVtPad;
   static constexpr size_t kQBytes = (size_t)kSp * AttnCfg<T>::kQkStride * sizeof(T);
-  static constexpr size_t kVtBytes = sizeof(T) == 2 ? (size_t)kSp * (kD + 16) * sizeof(T) : (size_t)kD * kVtStride * sizeof(T);
+  static constexpr size_t kVtBytes =
+      sizeof(T) == 2 ? (size_t)kSp * AttnCfg<_Float16>::kVStride * sizeof(T) : (size_t)kD * kVtStride * sizeof(T);
   static constexpr size_t kBytes = 2 * kQBytes + kVtBytes + kSp * sizeof(int);
 };
 
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   using C = Chunk16<T>;
   constexpr int kQS = Cfg::kQkStride;
   constexpr int kVS = Sm::kVtStride;
-  constexpr int kVR = kD + 16;                // fp16: stride of the row-major V tile (AttnCfg<_Float16>::kVStride)
+  constexpr int kVR = AttnCfg<_Float16>::kVStride;   // fp16: stride of the row-major V tile
   constexpr int kSp = Sm::kSp;
   constexpr int kCpr = kD / C::kElems;       // 16-byte chunks per head row
   constexpr int QPW = NKT > 4 ? NKT / 4 : 1; // query tiles per wavefront
@@ -535,7 +536,7 @@ constexpr int kLongChunk = kLongChunkTiles * 16;
 template <typename T>
 struct LongSmem {
   static constexpr int kQS = AttnCfg<T>::kQkStride;
-  static constexpr int kVR = kD + 16;                                  // fp16 V rows
+  static constexpr int kVR = AttnCfg<_Float16>::kVStride;              // fp16 V rows
   static constexpr int kVS = kLongChunk + AttnCfg<T>::kVtPad;          // fp32 V^T rows
   static constexpr size_t kKBytes = (size_t)kLongChunk * kQS * sizeof(T);
   static constexpr size_t kVBytes = sizeof(T) == 2 ? (size_t)kLongChunk * kVR * sizeof(T) : (size_t)kD * kVS * sizeof(T);

@@ -43,7 +43,15 @@ constexpr int kXcds = 8;
 
 // Workgroups are dealt round-robin to the 8 XCDs; give every XCD a contiguous band of tiles so that
 // the A rows a band shares stay in that XCD's L2.
-__device__ __forceinline__ int remap_tile(int pid, int per_xcd) { return (pid % kXcds) * per_xcd + pid / kXcds; }
+// The banding runs over the tiles that hold valid rows only (`valid_tiles`, a prefix of the tile order): with the row
+// count known on the device alone the launch covers every possible tile, and bands cut from all of them would leave
+// the last XCDs nothing but empty tiles.  Returns -1 for a workgroup without a tile.
+__device__ __forceinline__ int remap_valid_tile(int pid, int valid_tiles) {
+  const int per_xcd = (valid_tiles + kXcds - 1) / kXcds;
+  const int slot = pid / kXcds;
+  const int tile = (pid % kXcds) * per_xcd + slot;
+  return slot < per_xcd && tile < valid_tiles ? tile : -1;
+}
 
 // ------------------------------------------------------------------------------------------
 // fp16: (32*MI) x 256 tile, 4 wavefronts (2x2), k-step 32 = one v_mfma_f32_16x16x32_f16 depth.
@@ -108,16 +116,15 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
   constexpr int BM = Tile::BM, BN = kHBN;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-  const int tile = remap_tile(blockIdx.x, args.per_xcd);
+  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
   const int tiles_n_all = args.tiles_n * args.groups;
-  if (tile >= args.tiles_m * tiles_n_all) return;
+  const int tile = remap_valid_tile(blockIdx.x, ((rows + BM - 1) / BM) * tiles_n_all);
+  if (tile < 0) return;
   const int tm = tile / tiles_n_all;
   const int tn_all = tile - tm * tiles_n_all;
   const int grp = tn_all / args.tiles_n;
   const int tn = tn_all - grp * args.tiles_n;
-  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
   const int m0 = tm * BM;
-  if (m0 >= rows) return;
   const int n0 = tn * BN;
   const int N = args.n, K = args.k;
 
@@ -272,7 +279,7 @@ constexpr int kPThreads = 512;
 constexpr int kPBM = 256, kPBN = 256;
 constexpr int kPStage = (kPBM * kHBK + kHBK * kPBN) * 2;      // 32 KB per k-step
 constexpr int kPSmem = kStages * kPStage;                     // 128 KB
-constexpr int kPABytes = kPBM * kHBK * 2;     // A part of a k-step slot, B follows
+[[maybe_unused]] constexpr int kPABytes = kPBM * kHBK * 2;     // A part of a k-step slot, B follows
 
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
@@ -505,16 +512,15 @@ constexpr size_t kFStage = kFABytes + kFBBytes;
 
 __global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kFStage];
-  const int tile = remap_tile(blockIdx.x, args.per_xcd);
+  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
   const int tiles_n_all = args.tiles_n * args.groups;
-  if (tile >= args.tiles_m * tiles_n_all) return;
+  const int tile = remap_valid_tile(blockIdx.x, ((rows + kFBM - 1) / kFBM) * tiles_n_all);
+  if (tile < 0) return;
   const int tm = tile / tiles_n_all;
   const int tn_all = tile - tm * tiles_n_all;
   const int grp = tn_all / args.tiles_n;
   const int tn = tn_all - grp * args.tiles_n;
-  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
   const int m0 = tm * kFBM;
-  if (m0 >= rows) return;
   const int n0 = tn * kFBN;
   const int N = args.n, K = args.k;
   const float* __restrict__ A = (const float*)args.A[grp];
