@@ -504,13 +504,19 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
 // fp32: 128x128x16 tile, 4 wavefronts (2x2) of 64x64, v_mfma_f32_32x32x2_f32
 // ------------------------------------------------------------------------------------------
 constexpr int kFThreads = 256;
-constexpr int kFBM = 128, kFBN = 128, kFBK = 16;
+constexpr int kFBK = 16;
 constexpr int kFAStride = kFBK + 4;       // floats; 80-byte rows
-constexpr size_t kFABytes = (size_t)kFBM * kFAStride * 4;
-constexpr size_t kFBBytes = (size_t)kFBK * kFBN * 4;
-constexpr size_t kFStage = kFABytes + kFBBytes;
 
+// WB = 32x32 MFMA blocks per wavefront and dimension: 2 -> 128x128 tile, 1 -> 64x64 tile (problems of less than a
+// round of 128x128 tiles, where the time is the k loop of one tile: a quarter of the MFMAs per k-step)
+template <int WB>
 __global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
+  constexpr int kFBM = 64 * WB, kFBN = 64 * WB;
+  constexpr size_t kFABytes = (size_t)kFBM * kFAStride * 4;
+  constexpr size_t kFBBytes = (size_t)kFBK * kFBN * 4;
+  constexpr size_t kFStage = kFABytes + kFBBytes;
+  constexpr int kBc4 = kFBN / 4;            // 16-byte pieces per k-row of the B tile
+  constexpr int kBRows = kFThreads / kBc4;  // k-rows one pass of the workgroup covers
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kFStage];
   const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
   const int tiles_n_all = args.tiles_n * args.groups;
@@ -532,36 +538,36 @@ __global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, kb = lane >> 5;
 
-  u32x4 ra[2], rb[2];
-  const int a_kc = tid & 3, a_row = tid >> 2;       // + u*64
-  const int b_nc = tid & 31, b_krow = tid >> 5;     // + u*8
+  u32x4 ra[WB], rb[WB];
+  const int a_kc = tid & 3, a_row = tid >> 2;                // + u*64
+  const int b_nc = tid % kBc4, b_krow = tid / kBc4;          // + u*kBRows
   const bool b_col_ok = n0 + b_nc * 4 < N;
 
   auto load_global = [&](int k0) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < WB; ++u) {
       const int row = m0 + a_row + u * 64;
       ra[u] = u32x4{0u, 0u, 0u, 0u};
       if (row < rows) ra[u] = *reinterpret_cast<const u32x4*>(A + (size_t)row * K + k0 + a_kc * 4);
       rb[u] = u32x4{0u, 0u, 0u, 0u};
-      if (b_col_ok) rb[u] = *reinterpret_cast<const u32x4*>(B + (size_t)(k0 + b_krow + u * 8) * N + n0 + b_nc * 4);
+      if (b_col_ok) rb[u] = *reinterpret_cast<const u32x4*>(B + (size_t)(k0 + b_krow + u * kBRows) * N + n0 + b_nc * 4);
     }
   };
   auto store_lds = [&](int stage) {
     float* As = reinterpret_cast<float*>(smem + stage * kFStage);
     float* Bs = reinterpret_cast<float*>(smem + stage * kFStage + kFABytes);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < WB; ++u) {
       *reinterpret_cast<u32x4*>(As + (a_row + u * 64) * kFAStride + a_kc * 4) = ra[u];
-      *reinterpret_cast<u32x4*>(Bs + (b_krow + u * 8) * kFBN + b_nc * 4) = rb[u];
+      *reinterpret_cast<u32x4*>(Bs + (b_krow + u * kBRows) * kFBN + b_nc * 4) = rb[u];
     }
   };
 
-  float16v acc[2][2];
+  float16v acc[WB][WB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -574,10 +580,10 @@ __global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
     const float* As = reinterpret_cast<const float*>(smem + (kt & 1) * kFStage);
     const float* Bs = reinterpret_cast<const float*>(smem + (kt & 1) * kFStage + kFABytes);
     // step s of the stage contracts k = kb*8 + s (the same choice for A and B)
-    float a[2][8], b[2][8];
+    float a[WB][8], b[WB][8];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const float* ap = As + (wm * 64 + i * 32 + l32) * kFAStride + kb * 8;
+    for (int i = 0; i < WB; ++i) {
+      const float* ap = As + (wm * 32 * WB + i * 32 + l32) * kFAStride + kb * 8;
       const float4v a0 = *reinterpret_cast<const float4v*>(ap);
       const float4v a1 = *reinterpret_cast<const float4v*>(ap + 4);
 #pragma unroll
@@ -587,30 +593,30 @@ __global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
       }
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WB; ++j)
 #pragma unroll
-      for (int s = 0; s < 8; ++s) b[j][s] = Bs[(kb * 8 + s) * kFBN + wn * 64 + j * 32 + l32];
+      for (int s = 0; s < 8; ++s) b[j][s] = Bs[(kb * 8 + s) * kFBN + wn * 32 * WB + j * 32 + l32];
 #pragma unroll
     for (int s = 0; s < 8; ++s)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WB; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
     if (kt + 1 < nk) store_lds((kt + 1) & 1);
     __syncthreads();
   }
 
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int col = n0 + wn * 64 + j * 32 + l32;
+  for (int j = 0; j < WB; ++j) {
+    const int col = n0 + wn * 32 * WB + j * 32 + l32;
     if (col >= N) continue;
     const float bias = args.bias[grp] ? ((const float*)args.bias[grp])[col] : 0.f;
     float* C = (float*)args.C + (size_t)grp * N + col;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WB; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * kb + (r & 3);
+        const int row = m0 + wm * 32 * WB + i * 32 + 8 * (r >> 2) + 4 * kb + (r & 3);
         if (row < rows) C[(size_t)row * args.ldc] = acc[i][j][r] + bias;
       }
   }
@@ -771,11 +777,15 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
       else launch_f16<4>(a, stream);
     }
   } else {
-    a.tiles_m = (m_bound + kFBM - 1) / kFBM;
-    a.tiles_n = (n + kFBN - 1) / kFBN;
+    // less than a round of 128x128 tiles: 64x64 tiles finish their k loop four times sooner
+    const long big = (long)((m_bound + 127) / 128) * ((n + 127) / 128) * g.groups;
+    const int bt = big <= device_cu_count() ? 64 : 128;
+    a.tiles_m = (m_bound + bt - 1) / bt;
+    a.tiles_n = (n + bt - 1) / bt;
     const int total = a.tiles_m * a.tiles_n * a.groups;
     a.per_xcd = (total + kXcds - 1) / kXcds;
-    gemm_f32_kernel<<<a.per_xcd * kXcds, kFThreads, 0, stream>>>(a);
+    if (bt == 64) gemm_f32_kernel<1><<<a.per_xcd * kXcds, kFThreads, 0, stream>>>(a);
+    else gemm_f32_kernel<2><<<a.per_xcd * kXcds, kFThreads, 0, stream>>>(a);
   }
 }
 
