@@ -183,3 +183,34 @@ def test_long_sequences_layer_against_oracle(dtype):
     w = dict(wl=wl, lens=lens, mask=mask, attr_mask=attr, x=x, weights=weights)
     got = run_encoder(w)
     _check(got, _oracle(w), mask, dtype)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_against_oracle(seed):
+    """One layer on randomly drawn shapes (sequence lengths that are not multiples of 4 or 16, one head, holes in the
+    mask, empty sequences, both element types) against the oracle."""
+    rng = np.random.RandomState(1000 + seed)
+    dtype = ["fp32", "fp16"][seed % 2]
+    B = int(rng.randint(1, 9))
+    S = int(rng.choice([1, 3, 7, 16, 17, 33, 50, 64, 65, 96, 127, 130, 200]))
+    heads = int(rng.choice([1, 2, 3, 12]))
+    print("random shape", seed, dtype, "B", B, "S", S, "heads", heads, flush=True)
+    wl = o.Workload("rnd", 1000 + seed, dtype, 1, B, S, heads, 64, 4 * heads * 64, 1, S + 1)
+    if seed % 3 == 0:
+        mask = (rng.rand(B, S) < 0.7).astype(np.int32)
+        if B > 1:
+            mask[rng.randint(0, B)] = 0                       # an empty sequence
+        attr = (rng.rand(B, S, S) < 0.8).astype(np.float32)   # an attention mask unrelated to the input mask
+    else:
+        lens = rng.randint(1, S + 1, size=B)
+        mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.int32)
+        attr = np.ascontiguousarray(np.broadcast_to(mask[:, None, :], (B, S, S))).astype(np.float32)
+    attr = o.rnd(attr, dtype)
+    x = o.rnd(rng.randn(B, S, wl.H), dtype)
+    weights = o.make_layer_weights(wl, rng, True)
+    w = dict(wl=wl, lens=None, mask=mask, attr_mask=attr, x=x, weights=weights)
+    got = run_encoder(w)
+    if mask.sum() == 0:
+        assert np.all(got == 0)
+        return
+    _check(got, _oracle(w), mask, dtype)
