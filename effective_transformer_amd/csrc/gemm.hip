@@ -679,7 +679,7 @@ struct TransposeArgs {
 constexpr int kTrTile = 64;
 constexpr int kTrStride = kTrTile + 8;    // halves; 144-byte rows keep the 16-byte row reads aligned
 
-__global__ __launch_bounds__(256) void transpose_weights_kernel(TransposeArgs args) {
+__global__ __launch_bounds__(256) void layer_prologue_kernel(TransposeArgs args) {
   __shared__ __attribute__((aligned(16))) _Float16 tile[kTrTile * kTrStride];
   if ((int)blockIdx.x >= args.tile_begin[TransposeJobs::kMax]) {
     const int T = args.seq.rows_dev ? min(*args.seq.rows_dev, args.seq.rows_bound) : args.seq.rows_bound;
@@ -740,7 +740,7 @@ void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, con
   for (int j = jobs.count; j <= TransposeJobs::kMax; ++j) a.tile_begin[j] = total;
   a.seq = seq ? *seq : SeqStartJob{nullptr, nullptr, 0, 0, nullptr};
   if (seq) total += (seq->rows_bound + 1 + 255) / 256;
-  transpose_weights_kernel<<<total, 256, 0, stream>>>(a);
+  layer_prologue_kernel<<<total, 256, 0, stream>>>(a);
 }
 
 bool gemm_supported(DType t, int n, int k, int groups) {
