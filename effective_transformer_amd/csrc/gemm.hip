@@ -510,7 +510,7 @@ constexpr int kFAStride = kFBK + 4;       // floats; 80-byte rows
 // WB = 32x32 MFMA blocks per wavefront and dimension: 2 -> 128x128 tile, 1 -> 64x64 tile (problems of less than a
 // round of 128x128 tiles, where the time is the k loop of one tile: a quarter of the MFMAs per k-step)
 template <int WB>
-__global__ __launch_bounds__(kFThreads) void gemm_f32_kernel(GemmArgs args) {
+__global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
   constexpr int kFBM = 64 * WB, kFBN = 64 * WB;
   constexpr size_t kFABytes = (size_t)kFBM * kFAStride * 4;
   constexpr size_t kFBBytes = (size_t)kFBK * kFBN * 4;
