@@ -20,6 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libet_hip.so")
+EXAMPLE = os.path.join(LIBDIR, "et_encoder_example")      # C++ host sample (csrc/encoder_example.cpp)
 
 SOURCES = ["input_output.hip", "row_kernels.hip", "attention.hip", "gemm.hip", "et_api.cpp"]
 
@@ -62,6 +63,12 @@ def build(force: bool = True, jobs: int = 4) -> str:
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
     os.replace(tmp, LIB)
+    # the C++ host sample links against the library it sits beside
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O2", "-std=c++17", os.path.join(CSRC, "encoder_example.cpp"), "-o", EXAMPLE,
+           "-L" + LIBDIR, "-let_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the C++ sample failed:\n%s\n%s" % (r.stdout, r.stderr))
     return LIB
 
 

@@ -214,3 +214,31 @@ def test_random_shapes_against_oracle(seed):
         assert np.all(got == 0)
         return
     _check(got, _oracle(w), mask, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_cpp_host_gives_the_same_bits(tmp_path, dtype):
+    """The C++ sample (csrc/encoder_example.cpp on include/et.hpp) against the Python mirror on the same problem."""
+    import os
+    import subprocess
+    from effective_transformer_amd import build as b
+    print("C++ host", dtype, flush=True)
+    if not os.path.exists(b.EXAMPLE):
+        pytest.fail("lib/et_encoder_example has not been built (python -m effective_transformer_amd.build)")
+    w = o.make_workload("cfg1" if dtype == "fp32" else "cfg2", layers=2, random_affine=True)
+    wl = w["wl"]
+    npdt = np.float32 if dtype == "fp32" else np.float16
+    prob, outp = str(tmp_path / "problem.bin"), str(tmp_path / "out.bin")
+    with open(prob, "wb") as f:
+        np.array([0 if dtype == "fp32" else 1, wl.B, wl.S, wl.heads, wl.d, 2], np.int32).tofile(f)
+        w["mask"].astype(np.int32).tofile(f)
+        w["x"].astype(npdt).tofile(f)
+        w["attr_mask"].astype(npdt).tofile(f)
+        for a in w["weights"][:32]:
+            np.ascontiguousarray(a).astype(npdt).tofile(f)
+    r = subprocess.run([b.EXAMPLE, prob, outp], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert "valid tokens %d of %d" % (int(w["mask"].sum()), wl.B * wl.S) in r.stdout
+    got = np.fromfile(outp, dtype=npdt).reshape(wl.B, wl.S, wl.H)
+    want = run_encoder(w, layers=2)
+    assert np.array_equal(got, want)
