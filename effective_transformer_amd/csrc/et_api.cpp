@@ -594,7 +594,7 @@ et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt,
   ET_REQUIRE(h, m >= 0 && n >= 1 && k >= 1, "bad dimensions");
   if ((uint64_t)m * k * 2 > 0xffffffffull) return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
   if (!et::gemm_takes_transposed_b(et::DType::F16, m, n, n, k, 1))
-    return fail(h, ET_UNSUPPORTED, "et_gemm_bt needs k % 32 == 0, n % 8 == 0 and at least 128 tiles of 256x256");
+    return fail(h, ET_UNSUPPORTED, "et_gemm_bt needs k % 64 == 0, n % 8 == 0 and at least 128 tiles of 256x256");
   et::GemmGroups g;
   g.groups = 1;
   g.A[0] = A; g.B[0] = Bt; g.bias[0] = bias;

@@ -261,7 +261,8 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
 }
 
 // ------------------------------------------------------------------------------------------
-// fp16, large problems: persistent 256 x 256 tiles, 8 wavefronts (two per SIMD) in opposite phases.
+// fp16, large problems, B in its [k][n] storage order: persistent 256 x 256 tiles, 8 wavefronts (two per SIMD) in
+// opposite phases.
 //
 // Wave tile 128 x 64 (32 MFMAs per k-step, 128 accumulator registers), so two wavefronts fit one SIMD.
 // Waves 0-3 and 4-7 alternate: while one group issues its 32 MFMAs (raised priority) the other does
@@ -287,7 +288,6 @@ struct PTile {
   int m0, n0, grp;
 };
 
-template <bool BT>
 __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -336,17 +336,10 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
       const int row = q * 16 + (lane >> 2);
       const int c = (lane & 3) ^ a_swizzle(row);
       s.off[j] = ((uint32_t)(t.m0 + row) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
-      if (BT) {
-        // B^T rows are columns of C.  LDS row j*16+l of a 64-column group holds column 4*l+j, so that the operand
-        // reads look like A's and a lane still owns 4 consecutive columns of C
-        const int col = min(t.n0 + (row & ~63) + (row & 15) * 4 + ((row >> 4) & 3), N - 1);   // beyond N: never stored
-        s.off[2 + j] = ((uint32_t)col * (uint32_t)K + (uint32_t)c * 8u) * 2u;
-      } else {
-        const int kr = q * 2 + (lane >> 5);
-        const int pc = ((lane & 31) - 8 * ((kr >> 3) & 1)) & 31;   // B rows 8..15, 24..31 are rotated by 128 bytes in LDS
-        const int col = min(t.n0 + pc * 8, N - 8);                 // columns beyond N: a valid column, never stored
-        s.off[2 + j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
-      }
+      const int kr = q * 2 + (lane >> 5);
+      const int pc = ((lane & 31) - 8 * ((kr >> 3) & 1)) & 31;   // B rows 8..15, 24..31 are rotated by 128 bytes in LDS
+      const int col = min(t.n0 + pc * 8, N - 8);                 // columns beyond N: a valid column, never stored
+      s.off[2 + j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
     }
     return s;
   };
@@ -360,7 +353,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
 #pragma unroll
     for (int j = 0; j < 2; ++j)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(s.b, ET_LDS_PTR(st + kPABytes + (wave * 2 + j) * 1024), 16, s.off[2 + j],
-                                               BT ? kt * kHBK * 2 : kt * kHBK * N * 2, 0, 0);
+                                               kt * kHBK * N * 2, 0, 0);
   };
 
   // LDS operand addresses: A row (wm*128 + i*16 + l16), chunk g (swizzled); B k-row g*8+kk, 4 columns
@@ -371,7 +364,6 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
     const int row = g * 8 + kk;
     b_rd[kk] = row * 512 + (((wn * 64 + l16 * 4) * 2 + 128 * ((row >> 3) & 1)) & 511);
   }
-  const int bt_rd = ((wn * 64 + l16) * 4 + (g ^ a_swizzle(l16))) * 16;   // B^T: row (wn*64 + j*16 + l16), chunk g
 
   int idx = blockIdx.x;
   if (!valid(idx)) return;
@@ -385,28 +377,21 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
   auto fetch_phase = [&](int kt_issue, const Src& s, bool check) {
     issue((u + 3) & 3, kt_issue, s);
     const unsigned char* st = smem + (u & 3) * kPStage;
-    if constexpr (BT) {
+    uint2v raw[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bop[j] = *reinterpret_cast<const half8*>(st + kPABytes + bt_rd + j * 16 * 64);
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint2v*>(st + kPABytes + b_rd[kk]);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
-    } else {
-      uint2v raw[8];
+    for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
 #pragma unroll
-      for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint2v*>(st + kPABytes + b_rd[kk]);
+    for (int jj = 0; jj < 2; ++jj) {             // 8(k) x 4(n) block -> 4 operands
+      uint4v lo, hi;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) a[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
-#pragma unroll
-      for (int jj = 0; jj < 2; ++jj) {           // 8(k) x 4(n) block -> 4 operands
-        uint4v lo, hi;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          lo[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x05040100u);
-          hi[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x07060302u);
-        }
-        bop[2 * jj] = __builtin_bit_cast(half8, lo);
-        bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
+      for (int p = 0; p < 4; ++p) {
+        lo[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x05040100u);
+        hi[p] = __builtin_amdgcn_perm(raw[2 * p + 1][jj], raw[2 * p][jj], 0x07060302u);
       }
+      bop[2 * jj] = __builtin_bit_cast(half8, lo);
+      bop[2 * jj + 1] = __builtin_bit_cast(half8, hi);
     }
     if (check) wait_vmcnt<8>();                // this wave's share of k-step u+1 has landed (u+2, u+3 may fly)
     wait_lgkmcnt0();
@@ -495,6 +480,211 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
   }
   if (phase_group == 0) barrier_only();        // matches the extra barrier the second group started with
   wait_vmcnt<0>();                             // no DMA may still target this workgroup's LDS when it ends
+#else
+  (void)args;
+#endif
+}
+
+// ------------------------------------------------------------------------------------------
+// fp16, large problems, B k-contiguous ([n][k], see launch_transpose_weights): persistent 256 x 256 tiles, 8 wavefronts
+// that each pipeline their own work, LDS slots of two k-steps.
+//
+// Both operands are fetched in rows of 64 k = 128 bytes, one full cache line per row: eight lanes of a DMA instruction
+// cover a line, where rows of 32 k leave every second half-line request to the next k-step.  Two such slots (2 x 64 KB)
+// make the ring.  A wave (tile 128 x 64, two operand register sets) reads the operands of k-step t+1 from LDS and
+// issues its share of the DMA for the pair after next between the MFMAs of k-step t, so no wave ever stops for a fetch
+// phase, and the only synchronisation is one barrier per pair of k-steps: after the even step every wave has read its
+// slot for the last time (the slot becomes the DMA target during the odd step) and this wave's share of the other slot
+// has landed.  The 16-byte chunks of a 128-byte LDS row are XOR-swizzled with row bits 1-3, which spreads the 16 rows
+// x one chunk of an MFMA operand read over all 64 banks.
+// A, B^T and C are addressed through per-tile buffer descriptors (base at the tile, records = what the matrix has
+// left there), so lane offsets are tile-independent, rows beyond the valid-token count read as zero and are dropped
+// on the way out, and no offset grows with the size of the matrices.
+// ------------------------------------------------------------------------------------------
+constexpr int kQAPair = kPBM * 128;                            // 32 KB: 256 rows x two k-steps
+constexpr int kQPair = kQAPair + kPBN * 128;                   // 64 KB: A rows, then B^T rows
+constexpr int kQSmem = 2 * kQPair;
+
+__device__ __forceinline__ int pair_swizzle(int row) { return (row >> 1) & 7; }
+
+__global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args) {
+#if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // 0..7, scalar
+  const int wm = wave & 1, wn = (wave >> 1) & 3;                  // 128-row half, 64-column quarter of the tile
+  const int l16 = lane & 15, g = lane >> 4;
+  const int N = args.n, K = args.k;
+  const int np = K / 64;                                          // pairs of k-steps per tile, >= 2
+
+  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
+  const int tiles_n_all = args.tiles_n * args.groups;
+  const int total = ((rows + kPBM - 1) / kPBM) * tiles_n_all;     // tiles that hold valid rows (a prefix in tile order)
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds;
+  const int G = gridDim.x;                                        // multiple of 8
+
+  auto tile_id = [&](int idx) { return xcd * per_xcd + idx / kXcds; };
+  auto valid = [&](int idx) { return idx / kXcds < per_xcd && tile_id(idx) < total; };
+
+  struct Src {
+    __amdgpu_buffer_rsrc_t a, b;
+    int m0, n0, grp;
+  };
+  auto locate = [&](int tile) {
+    Src t;
+    if (args.reverse_walk) tile = total - 1 - tile;
+    const int tm = tile / tiles_n_all;
+    const int tn_all = tile - tm * tiles_n_all;
+    t.grp = tn_all / args.tiles_n;
+    t.m0 = tm * kPBM;
+    t.n0 = (tn_all - t.grp * args.tiles_n) * kPBN;
+    t.a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16*>((const _Float16*)args.A[t.grp] + (size_t)t.m0 * K), 0, min(rows - t.m0, kPBM) * K * 2, 0x00020000);
+    t.b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16*>((const _Float16*)args.B[t.grp] + (size_t)t.n0 * K), 0, min(N - t.n0, kPBN) * K * 2, 0x00020000);
+    return t;
+  };
+
+  // DMA: one instruction fills 1 KB of LDS = 8 rows x 128 bytes.  This wave owns rows wave*32 .. wave*32+31 of the A
+  // part and of the B^T part of a slot (4 + 4 instructions per pair).  LDS row j*16+l of a 64-column group holds
+  // column 4*l+j of the tile, so that the operand reads of B^T look like A's and a lane owns 4 consecutive columns of C.
+  uint32_t voff_a[4], voff_b[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = wave * 32 + j * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ pair_swizzle(row);
+    voff_a[j] = ((uint32_t)row * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+    const int col = (row & ~63) + (row & 15) * 4 + ((row >> 4) & 3);
+    voff_b[j] = ((uint32_t)col * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+  }
+  // instruction q (0..3: A, 4..7: B^T) of this wave's share of pair `pr` of a tile into slot `slot`
+  auto issue1 = [&](int slot, int pr, const __amdgpu_buffer_rsrc_t& ra, const __amdgpu_buffer_rsrc_t& rb, int q) {
+    unsigned char* st = smem + slot * kQPair;
+    if (q < 4)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, ET_LDS_PTR(st + (wave * 4 + q) * 1024), 16, voff_a[q], pr * 128, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, ET_LDS_PTR(st + kQAPair + (wave * 4 + q - 4) * 1024), 16,
+                                               voff_b[q - 4], pr * 128, 0, 0);
+  };
+
+  // operand reads: row (wm*128 + i*16 + l16) resp. (wn*64 + j*16 + l16), chunk (4*half + g), swizzled
+  const int sw = pair_swizzle(l16);
+  const int a_rd[2] = {(wm * 128 + l16) * 128 + ((g ^ sw) * 16), (wm * 128 + l16) * 128 + (((4 + g) ^ sw) * 16)};
+  const int b_rd[2] = {kQAPair + (wn * 64 + l16) * 128 + ((g ^ sw) * 16),
+                       kQAPair + (wn * 64 + l16) * 128 + (((4 + g) ^ sw) * 16)};
+
+  int idx = blockIdx.x;
+  if (!valid(idx)) return;
+  Src cur = locate(tile_id(idx)), nxt = cur;
+
+  float4v acc[8][4];
+  half8 a[2][8], b[2][4];
+  int pairs_done = 0;                            // by this workgroup: slot of a pair = pairs_done & 1
+
+  // One k-step: MFMAs on operand set P; half `rh` of slot `rs` is read into the other set; with DMA set, this wave's
+  // eight DMA instructions for pair `dpr` (descriptors da, db) go into slot `ds`, one after each group of four MFMAs.
+  auto step = [&](auto Pc, auto FIRSTc, auto DMAc, int rs, int ds, int dpr, const __amdgpu_buffer_rsrc_t& da,
+                  const __amdgpu_buffer_rsrc_t& db) {
+    constexpr int P = decltype(Pc)::value;
+    constexpr bool FIRST = decltype(FIRSTc)::value;
+    constexpr bool DMA = decltype(DMAc)::value;
+    constexpr int rh = 1 - P;                    // the even step reads half 1 of its own pair, the odd step half 0 of the next
+    const unsigned char* ns = smem + rs * kQPair;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i < 2) {
+        b[1 - P][2 * i] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + (2 * i) * 2048);
+        b[1 - P][2 * i + 1] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + (2 * i + 1) * 2048);
+      } else if (i < 6) {
+        a[1 - P][2 * (i - 2)] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (2 * (i - 2)) * 2048);
+        a[1 - P][2 * (i - 2) + 1] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (2 * (i - 2) + 1) * 2048);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[P][i], b[P][j],
+                                                           FIRST ? float4v{0.f, 0.f, 0.f, 0.f} : acc[i][j], 0, 0, 0);
+      if (DMA) issue1(ds, dpr, da, db, i);
+      __builtin_amdgcn_sched_barrier(0);         // keeps the reads and the DMA where they are between the MFMA groups
+    }
+  };
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+
+  // pairs 0 and 1 of the first tile, operands of k-step 0
+#pragma unroll
+  for (int q = 0; q < 8; ++q) issue1(0, 0, cur.a, cur.b, q);
+#pragma unroll
+  for (int q = 0; q < 8; ++q) issue1(1, 1, cur.a, cur.b, q);
+  wait_vmcnt<8>();
+  barrier_only();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const half8*>(smem + b_rd[0] + j * 2048);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[0][i] = *reinterpret_cast<const half8*>(smem + a_rd[0] + i * 2048);
+
+  bool first_tile = true;
+  while (true) {
+    const int nidx = idx + G;
+    const bool has_next = valid(nidx);
+    if (has_next) nxt = locate(tile_id(nidx));   // otherwise the stream re-loads this tile; the data is never used
+    for (int p = 0; p < np; ++p) {
+      const int s = pairs_done & 1;
+      if (p == 0) step(Even{}, std::true_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
+      else step(Even{}, std::false_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
+      // this wave's share of the next pair has landed (right after a tile boundary that was confirmed before the C
+      // stores went out) and its last reads of slot s, which feed the odd step, are complete
+      if (first_tile || p >= 1) wait_vmcnt<0>();
+      wait_lgkmcnt0();
+      barrier_only();
+      // pair p+2 of this tile, or the matching pair of the next one, replaces slot s
+      const bool in_tile = p + 2 < np;
+      const __amdgpu_buffer_rsrc_t da = in_tile ? cur.a : nxt.a;
+      const __amdgpu_buffer_rsrc_t db = in_tile ? cur.b : nxt.b;
+      step(Odd{}, std::false_type{}, std::true_type{}, s ^ 1, s, in_tile ? p + 2 : p + 2 - np, da, db);
+      ++pairs_done;
+    }
+    wait_vmcnt<0>();
+    {
+      // C leaves through a descriptor that covers the tile's valid rows only: rows beyond them are dropped by the
+      // bounds check, and the only per-store address arithmetic is one add on the running byte offset
+      const int col = cur.n0 + wn * 64 + l16 * 4;
+      if (col < N) {
+        const int tile_rows = min(rows - cur.m0, kPBM), tile_cols = min(N - cur.n0, kPBN);
+        _Float16* cbase = (_Float16*)args.C + (size_t)cur.m0 * args.ldc + (size_t)cur.grp * N + cur.n0;
+        const __amdgpu_buffer_rsrc_t rc =
+            __builtin_amdgcn_make_buffer_rsrc(cbase, 0, ((tile_rows - 1) * args.ldc + tile_cols) * 2, 0x00020000);
+        const uint32_t row_bytes = (uint32_t)args.ldc * 2u;
+        uint32_t voff = ((uint32_t)(wm * 128 + g * 4) * (uint32_t)args.ldc + (uint32_t)(wn * 64 + l16 * 4)) * 2u;
+        // the offset is the same for every tile; the empty asm keeps the compiler from computing all 32 store offsets
+        // once and holding them in registers across the k loop
+        asm volatile("" : "+v"(voff));
+        // bias added in half on the rounded product, as the reference's next kernel does; without a bias the addend is
+        // -0, which leaves every value (and the sign of a zero) as it is
+        half4 bias4 = {(_Float16)-0.0f, (_Float16)-0.0f, (_Float16)-0.0f, (_Float16)-0.0f};
+        if (args.bias[cur.grp] != nullptr) bias4 = *reinterpret_cast<const half4*>((const _Float16*)args.bias[cur.grp] + col);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            half4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = f2h(acc[i][j][r]);
+            o = o + bias4;
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, o), rc, voff, 0, 2 /* nt */);
+            voff += row_bytes;
+          }
+          voff += 12u * row_bytes;
+        }
+      }
+    }
+    if (!has_next) break;
+    idx = nidx;
+    cur = nxt;
+    first_tile = false;
+  }
+  wait_vmcnt<0>();                               // no DMA may still target this workgroup's LDS when it ends
 #else
   (void)args;
 #endif
@@ -646,9 +836,9 @@ int device_cu_count() {
   return cus[dev];
 }
 
-template <bool BT>
-void launch_f16_persistent(GemmArgs a, hipStream_t stream) {
-  allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel<BT>), kPSmem);
+void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
+  if (b_transposed) allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_pair_kernel), kQSmem);
+  else allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel), kPSmem);
   a.tiles_m = (a.m_bound + kPBM - 1) / kPBM;
   a.tiles_n = (a.n + kPBN - 1) / kPBN;
   const int total = a.tiles_m * a.tiles_n * a.groups;
@@ -658,7 +848,8 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream) {
   // k > n: A is the big operand and was written front to back by the kernel before this one, so its last rows are the
   // ones most likely still in the last-level cache: walk the tiles from the end
   a.reverse_walk = a.k > a.n ? 1 : 0;
-  gemm_f16_persistent_kernel<BT><<<grid, kPThreads, kPSmem, stream>>>(a);
+  if (b_transposed) gemm_f16_pair_kernel<<<grid, kPThreads, kQSmem, stream>>>(a);
+  else gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
 }
 
 // few big tiles would leave most of the 256 CUs idle: the persistent 256x256 kernel only runs when there is work
@@ -719,11 +910,12 @@ __global__ __launch_bounds__(256) void layer_prologue_kernel(TransposeArgs args)
 }  // namespace
 
 bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
-  return t == DType::F16 && gemm_supported(t, n, k, groups) && k % 8 == 0 && use_persistent(m_bound, ldc, n, k, groups);
+  return t == DType::F16 && gemm_supported(t, n, k, groups) && k % 64 == 0 && use_persistent(m_bound, ldc, n, k, groups);
 }
 
 // Inside the layer the transposed copy pays off for the wide projections (QKV, FFN up: many column tiles re-read a
-// short k extent); with k > n the [k][n] rows of 512 contiguous bytes are the better fetch and the copy is skipped.
+// short k extent).  With k >= n the activations stream through L2 once per few tiles and the [k][n] kernel, whose B rows
+// are 512 contiguous bytes, is as fast inside the layer as the k-contiguous one is on its own, so the copy is skipped.
 bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
   return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && (long)n * groups >= 2L * k;
 }
@@ -767,8 +959,7 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.groups = g.groups;
   if (t == DType::F16) {
     if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
-      if (g.b_transposed) launch_f16_persistent<true>(a, stream);
-      else launch_f16_persistent<false>(a, stream);
+      launch_f16_persistent(a, stream, g.b_transposed);
     } else {
       // less than a round of tiles: the time is the latency of one tile's k loop, which is shorter for 64-row tiles
       // (two of their workgroups fit a CU); from about two tiles per CU on the 128-row tile is the better one

@@ -235,7 +235,8 @@ et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void
 
 /* et_gemm with the second operand k-contiguous: C[m,n] = A[m,k] . Bt[n,k]^T (+ bias), fp16 only.  This is the kernel
  * et_layer runs once a batch has enough tokens to fill the chip (same cublasGemmEx call sites as et_gemm);
- * ET_UNSUPPORTED for shapes with fewer than 128 tiles of 256x256, which go through et_gemm's kernels. */
+ * ET_UNSUPPORTED for k % 64 != 0 and for shapes with fewer than 128 tiles of 256x256, which go through et_gemm's
+ * kernels. */
 et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
                      int m, int n, int k, const int32_t* m_dev, void* stream);
 
