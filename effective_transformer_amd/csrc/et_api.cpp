@@ -349,8 +349,12 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   // FFN up + bias + GELU (:215-227)
   g1.A[0] = attn; g1.B[0] = t_up ? wt_up : w->inter_kernel;
   g1.b_transposed = t_up;
+  // the large-M kernel applies bias + GELU to its tile on the way out; elsewhere it is a pass of its own
+  const bool fused_gelu = et::gemm_fuses_bias_gelu(dt, rows, F, F, H, 1, t_up);
+  if (fused_gelu) { g1.bias[0] = w->inter_bias; g1.gelu = true; }
   et::launch_gemm(dt, g1, inter, F, rows, F, H, T, st);
-  et::launch_bias_gelu(dt, inter, w->inter_bias, rows, F, T, st);
+  if (!fused_gelu) et::launch_bias_gelu(dt, inter, w->inter_bias, rows, F, T, st);
+  g1.bias[0] = nullptr; g1.gelu = false;
   if ((s = check_launch(h, "FFN up")) != ET_OK) return s;
   // FFN down + bias + residual(LN1 output) + LayerNorm (:229-247)
   g1.A[0] = inter; g1.B[0] = t_down ? wt_down : w->output_kernel;
@@ -584,23 +588,40 @@ et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void
   return check_launch(h, "weight transpose");
 }
 
-et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias, int m, int n,
-                     int k, const int32_t* m_dev, void* stream) {
+namespace {
+
+et_status gemm_bt_impl(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias, int m, int n,
+                       int k, const int32_t* m_dev, void* stream, bool gelu, const char* what) {
   et_status s = enter(h);
   if (s != ET_OK) return s;
   Scope scope(h);
   ET_REQUIRE(h, dtype == ET_FP16, "dtype must be ET_FP16");
   ET_REQUIRE(h, A && Bt && C, "null tensor pointer");
+  ET_REQUIRE(h, !gelu || bias, "null bias");
   ET_REQUIRE(h, m >= 0 && n >= 1 && k >= 1, "bad dimensions");
   if ((uint64_t)m * k * 2 > 0xffffffffull) return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
   if (!et::gemm_takes_transposed_b(et::DType::F16, m, n, n, k, 1))
-    return fail(h, ET_UNSUPPORTED, "et_gemm_bt needs k % 64 == 0, n % 8 == 0 and at least 128 tiles of 256x256");
+    return fail(h, ET_UNSUPPORTED,
+                std::string(what) + " needs k % 64 == 0, n % 8 == 0 and at least 128 tiles of 256x256");
   et::GemmGroups g;
   g.groups = 1;
   g.A[0] = A; g.B[0] = Bt; g.bias[0] = bias;
   g.b_transposed = true;
+  g.gelu = gelu;
   et::launch_gemm(et::DType::F16, g, C, n, m, n, k, m_dev, (hipStream_t)stream);
-  return check_launch(h, "gemm_bt");
+  return check_launch(h, what);
+}
+
+}  // namespace
+
+et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias, int m, int n,
+                     int k, const int32_t* m_dev, void* stream) {
+  return gemm_bt_impl(h, dtype, A, Bt, C, bias, m, n, k, m_dev, stream, false, "et_gemm_bt");
+}
+
+et_status et_gemm_bt_bias_gelu(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
+                               int m, int n, int k, const int32_t* m_dev, void* stream) {
+  return gemm_bt_impl(h, dtype, A, Bt, C, bias, m, n, k, m_dev, stream, true, "et_gemm_bt_bias_gelu");
 }
 
 }  // extern "C"

@@ -115,6 +115,26 @@ __device__ __forceinline__ uint32_t div_by(uint32_t n, const fastdiv& f) {
 __device__ __forceinline__ float h2f(_Float16 h) { return (float)h; }
 __device__ __forceinline__ _Float16 f2h(float f) { return (_Float16)f; }   // v_cvt_f16_f32, round-to-nearest-even
 
+// ---- bias + GELU arithmetic (reference: cuda/cuda_kernels.cu:29-51) -------------------------
+// 0.5*(1+tanh(u)) is evaluated as 1/(1+exp(-2u)), which is the same function without the cancellation of 1+tanh for
+// negative u.
+__device__ __forceinline__ float gelu_cdf(float x, float x3) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x3);
+  const float e = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);      // exp(-2u) = 2^(-2u*log2(e))
+  return __builtin_amdgcn_rcpf(1.0f + e);
+}
+// fp16 rounding points of the reference: __hadd2 for the bias, two __hmul2 for the cube, the CDF in float rounded to
+// half, __hmul2.  HV is a vector of halves (half4, half8).
+template <typename HV, int N>
+__device__ __forceinline__ HV bias_gelu_half(HV v, HV bias) {
+  const HV x = v + bias;
+  const HV x3 = x * (x * x);
+  HV cdf;
+#pragma unroll
+  for (int i = 0; i < N; ++i) cdf[i] = f2h(gelu_cdf(h2f(x[i]), h2f(x3[i])));
+  return x * cdf;
+}
+
 // seq_start[b] = first packed row of sequence b (b in [0, batch]; seq_start[batch] = T), written by the thread that
 // owns packed row t in [0, T]: it covers the sequences that begin at t (token-less sequences included).
 __device__ __forceinline__ void seq_start_for_row(const int32_t* __restrict__ batch_idx, int T, int t, int batch,

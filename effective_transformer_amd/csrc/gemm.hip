@@ -35,6 +35,7 @@ struct GemmArgs {
   int tiles_m, tiles_n;      // tiles_n per group
   int per_xcd;               // workgroups per XCD slot of the launch
   int reverse_walk = 0;      // persistent kernel: walk the tiles from the last one
+  int gelu = 0;              // k-contiguous-B kernel: C = gelu(A.B + bias) instead of A.B + bias
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -507,6 +508,7 @@ constexpr int kQSmem = 2 * kQPair;
 
 __device__ __forceinline__ int pair_swizzle(int row) { return (row >> 1) & 7; }
 
+template <bool GELU>
 __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -671,7 +673,8 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
             half4 o;
 #pragma unroll
             for (int j = 0; j < 4; ++j) o[j] = f2h(acc[i][j][r]);
-            o = o + bias4;
+            // GELU here costs no pass over C: its arithmetic runs while the stores of the tile drain
+            o = GELU ? bias_gelu_half<half4, 4>(o, bias4) : o + bias4;
             __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, o), rc, voff, 0, 2 /* nt */);
             voff += row_bytes;
           }
@@ -837,7 +840,8 @@ int device_cu_count() {
 }
 
 void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
-  if (b_transposed) allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_pair_kernel), kQSmem);
+  if (b_transposed && a.gelu) allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_pair_kernel<true>), kQSmem);
+  else if (b_transposed) allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_pair_kernel<false>), kQSmem);
   else allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel), kPSmem);
   a.tiles_m = (a.m_bound + kPBM - 1) / kPBM;
   a.tiles_n = (a.n + kPBN - 1) / kPBN;
@@ -848,7 +852,8 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
   // k > n: A is the big operand and was written front to back by the kernel before this one, so its last rows are the
   // ones most likely still in the last-level cache: walk the tiles from the end
   a.reverse_walk = a.k > a.n ? 1 : 0;
-  if (b_transposed) gemm_f16_pair_kernel<<<grid, kPThreads, kQSmem, stream>>>(a);
+  if (b_transposed && a.gelu) gemm_f16_pair_kernel<true><<<grid, kPThreads, kQSmem, stream>>>(a);
+  else if (b_transposed) gemm_f16_pair_kernel<false><<<grid, kPThreads, kQSmem, stream>>>(a);
   else gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
 }
 
@@ -920,6 +925,10 @@ bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int 
   return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && (long)n * groups >= 2L * k;
 }
 
+bool gemm_fuses_bias_gelu(DType t, int m_bound, int ldc, int n, int k, int groups, bool b_transposed) {
+  return b_transposed && gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups);
+}
+
 void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, const SeqStartJob* seq) {
   if (jobs.count == 0 && seq == nullptr) return;
   TransposeArgs a;
@@ -957,6 +966,7 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.n = n;
   a.k = k;
   a.groups = g.groups;
+  a.gelu = g.gelu ? 1 : 0;        // only where gemm_fuses_bias_gelu() holds; the other kernels ignore it
   if (t == DType::F16) {
     if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
       launch_f16_persistent(a, stream, g.b_transposed);

@@ -12,16 +12,8 @@ namespace et {
 namespace {
 
 // ------------------------------------------------------------------------------------------
-// bias + GELU.  0.5*(1+tanh(u)) is evaluated as 1/(1+exp(-2u)), which is the same function
-// without the cancellation of 1+tanh for negative u.
+// bias + GELU (arithmetic in et_device.hpp, shared with the GEMM epilogue that fuses it)
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_cdf(float x, float x3) {
-  const float u = 0.7978845608028654f * (x + 0.044715f * x3);
-  // exp(-2u) = 2^(-2u*log2(e))
-  const float e = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);
-  return __builtin_amdgcn_rcpf(1.0f + e);
-}
-
 constexpr int kGeluThreads = 128;
 constexpr int kGeluRows = 16;     // rows per workgroup
 constexpr int kGeluInFlight = 4;  // rows loaded before any is computed
@@ -42,12 +34,7 @@ template <> struct GeluChunk<float> {
 template <> struct GeluChunk<_Float16> {
   half8 v;
   __device__ __forceinline__ void apply(const GeluChunk<_Float16>& b) {
-    const half8 x = v + b.v;                 // __hadd2
-    const half8 x3 = x * (x * x);            // two half roundings (__hmul2 twice)
-    half8 cdf;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) cdf[i] = f2h(gelu_cdf(h2f(x[i]), h2f(x3[i])));
-    v = x * cdf;
+    v = bias_gelu_half<half8, 8>(v, b.v);
   }
 };
 

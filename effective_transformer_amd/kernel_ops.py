@@ -119,12 +119,13 @@ def transpose_weight(w, out: Optional[torch.Tensor] = None):
 
 
 def gemm_bt(a, bt, bias=None, m: Optional[int] = None, m_dev: Optional[torch.Tensor] = None,
-            out: Optional[torch.Tensor] = None):
-    """a [m, k] . bt [n, k]^T: the large-M kernel of the encoder layer."""
+            out: Optional[torch.Tensor] = None, gelu: bool = False):
+    """a [m, k] . bt [n, k]^T (+ bias): the large-M kernel of the encoder layer.  gelu=True applies bias + GELU to the
+    product on its way out (what add_bias_act would do in a second pass)."""
     rows, k = a.shape
     n = bt.shape[0]
     if out is None:
         out = torch.zeros(rows, n, dtype=a.dtype, device=a.device)
-    _call("et_gemm_bt", a.device, _dtype_code(a.dtype), _p(a), _p(bt), _p(out), _p(bias), rows if m is None else m, n,
-          k, _p(m_dev), _stream())
+    _call("et_gemm_bt_bias_gelu" if gelu else "et_gemm_bt", a.device, _dtype_code(a.dtype), _p(a), _p(bt), _p(out),
+          _p(bias), rows if m is None else m, n, k, _p(m_dev), _stream())
     return out

@@ -240,6 +240,14 @@ et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void
 et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
                      int m, int n, int k, const int32_t* m_dev, void* stream);
 
+/* C[m,n] = gelu(A[m,k] . Bt[n,k]^T + bias[n]): et_gemm_bt with et_add_bias_act applied to each tile on its way out,
+ * same arithmetic and rounding points as the two calls in a row (reference: the cublasGemmEx call and the
+ * add_bias_act launch that follows it, tf_op/bert_transformer_op.cu.cc:215-227, cuda/cuda_kernels.cu:29-51, 88-150).
+ * This is what et_layer runs for the first FFN projection of a large batch.  fp16 only, bias required; shapes as
+ * for et_gemm_bt. */
+et_status et_gemm_bt_bias_gelu(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
+                               int m, int n, int k, const int32_t* m_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

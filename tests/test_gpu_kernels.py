@@ -345,6 +345,28 @@ def test_gemm_bt(k, m, n, k_):
     assert np.array_equal(got2[:m - 301], got[:m - 301]) and np.all(got2[m - 301:] == 0)
 
 
+@pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (5000, 3072, 768)])
+def test_gemm_bt_bias_gelu_equals_the_two_passes(k, m, n, k_):
+    print("gemm_bt_bias_gelu", m, n, k_, flush=True)
+    rng = np.random.RandomState(m + n + k_ + 1)
+    a = o.rnd(rng.randn(m, k_), "fp16")
+    b = o.rnd(0.05 * rng.randn(k_, n), "fp16")
+    bias = o.rnd(rng.randn(n), "fp16")
+    bt = k.transpose_weight(dev(b))
+    two = k.add_bias_act(k.gemm_bt(dev(a), bt), dev(bias)).cpu().numpy()
+    one = k.gemm_bt(dev(a), bt, bias=dev(bias), gelu=True).cpu().numpy()
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16))        # same rounding points, bit for bit
+    # against the oracle's bias + GELU on the product the kernel produced
+    prod = k.gemm_bt(dev(a), bt).cpu().numpy()
+    want = o.add_bias_act(prod, bias, "fp16")
+    assert np.max(np.abs(one.astype(np.float32) - want.astype(np.float32))) <= 2e-3 * max(1.0, np.abs(want).max())
+    md = torch.tensor([m - 301], dtype=torch.int32, device="cuda")
+    part = k.gemm_bt(dev(a), bt, bias=dev(bias), m_dev=md, gelu=True).cpu().numpy()
+    assert np.array_equal(part[:m - 301], one[:m - 301]) and np.all(part[m - 301:] == 0)
+    with pytest.raises(Exception, match="null bias"):
+        k.gemm_bt(dev(a), bt, gelu=True)
+
+
 def test_gemm_bt_small_shapes_are_refused(k):
     a = torch.zeros(1000, 768, dtype=torch.float16, device="cuda")
     bt = torch.zeros(768, 768, dtype=torch.float16, device="cuda")
