@@ -70,6 +70,7 @@ SIGNATURES = {
     "et_transpose_rm_padding": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "et_attention": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _sz, _vp]),
     "et_gemm": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "et_gemm_bias_gelu": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_transpose_weight": (_i, [_vp, _i, _vp, _vp, _i, _i, _vp]),
     "et_gemm_bt": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_gemm_bt_bias_gelu": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),

@@ -346,14 +346,12 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   et::launch_bias_residual_layernorm(dt, attn, from_tensor, w->attr_output_bias, w->attr_output_layernorm_gamma,
                                      w->attr_output_layernorm_beta, rows, H, T, st);
   if ((s = check_launch(h, "attention output")) != ET_OK) return s;
-  // FFN up + bias + GELU (:215-227)
+  // FFN up + bias + GELU (:215-227, cuda/cuda_kernels.cu:88-150)
   g1.A[0] = attn; g1.B[0] = t_up ? wt_up : w->inter_kernel;
   g1.b_transposed = t_up;
-  // the large-M kernel applies bias + GELU to its tile on the way out; elsewhere it is a pass of its own
-  const bool fused_gelu = et::gemm_fuses_bias_gelu(dt, rows, F, F, H, 1, t_up);
-  if (fused_gelu) { g1.bias[0] = w->inter_bias; g1.gelu = true; }
+  // bias + GELU are applied to each tile on its way out of the GEMM: no pass of its own over [T,4H]
+  g1.bias[0] = w->inter_bias; g1.gelu = true;
   et::launch_gemm(dt, g1, inter, F, rows, F, H, T, st);
-  if (!fused_gelu) et::launch_bias_gelu(dt, inter, w->inter_bias, rows, F, T, st);
   g1.bias[0] = nullptr; g1.gelu = false;
   if ((s = check_launch(h, "FFN up")) != ET_OK) return s;
   // FFN down + bias + residual(LN1 output) + LayerNorm (:229-247)
@@ -554,16 +552,19 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
   return check_launch(h, "attention");
 }
 
-et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias, int m, int n,
-                  int k, const int32_t* m_dev, void* stream) {
+namespace {
+
+et_status gemm_impl(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias, int m, int n,
+                    int k, const int32_t* m_dev, void* stream, bool gelu, const char* what) {
   et_status s = enter(h);
   if (s != ET_OK) return s;
   Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   ET_REQUIRE(h, A && B && C, "null tensor pointer");
+  ET_REQUIRE(h, !gelu || bias, "null bias");
   ET_REQUIRE(h, m >= 0 && n >= 1 && k >= 1, "bad dimensions");
   if (!et::gemm_supported(to_dt(dtype), n, k, 1))
-    return fail(h, ET_UNSUPPORTED, dtype == ET_FP16 ? "fp16 GEMM needs k % 64 == 0 and n % 8 == 0"
+    return fail(h, ET_UNSUPPORTED, dtype == ET_FP16 ? "fp16 GEMM needs k % 32 == 0 and n % 8 == 0"
                                                      : "fp32 GEMM needs k % 16 == 0 and n % 4 == 0");
   if ((uint64_t)m * k * et::elem_size(to_dt(dtype)) > 0xffffffffull)
     return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
@@ -571,8 +572,21 @@ et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, voi
   et::GemmGroups g;
   g.groups = 1;
   g.A[0] = A; g.B[0] = B; g.bias[0] = bias;
+  g.gelu = gelu;
   et::launch_gemm(to_dt(dtype), g, C, n, m, n, k, m_dev, (hipStream_t)stream);
-  return check_launch(h, "gemm");
+  return check_launch(h, what);
+}
+
+}  // namespace
+
+et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias, int m, int n,
+                  int k, const int32_t* m_dev, void* stream) {
+  return gemm_impl(h, dtype, A, B, C, bias, m, n, k, m_dev, stream, false, "gemm");
+}
+
+et_status et_gemm_bias_gelu(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias, int m,
+                            int n, int k, const int32_t* m_dev, void* stream) {
+  return gemm_impl(h, dtype, A, B, C, bias, m, n, k, m_dev, stream, true, "gemm + bias + gelu");
 }
 
 et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void* dst, int k, int n, void* stream) {

@@ -35,7 +35,7 @@ struct GemmArgs {
   int tiles_m, tiles_n;      // tiles_n per group
   int per_xcd;               // workgroups per XCD slot of the launch
   int reverse_walk = 0;      // persistent kernel: walk the tiles from the last one
-  int gelu = 0;              // k-contiguous-B kernel: C = gelu(A.B + bias) instead of A.B + bias
+  int gelu = 0;              // C = gelu(A.B + bias) instead of A.B + bias (bias must be set)
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -251,7 +251,9 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
           half8 o;
 #pragma unroll
           for (int j = 0; j < 8; ++j) o[j] = f2h(acc[i][j][r]);
-          if (has_bias) o = o + bias8;      // half add on the rounded product, as the reference's next kernel does
+          // half add on the rounded product, as the reference's next kernel does; optionally that kernel's GELU too
+          if (args.gelu) o = bias_gelu_half<half8, 8>(o, bias8);
+          else if (has_bias) o = o + bias8;
           __builtin_nontemporal_store(o, reinterpret_cast<half8*>(C + (size_t)row * args.ldc));
         }
       }
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
             __builtin_amdgcn_make_buffer_rsrc(args.C, 0, (int)((uint32_t)rows * (uint32_t)args.ldc * 2u), 0x00020000);
         const uint32_t row_bytes = (uint32_t)args.ldc * 2u;
         uint32_t voff = ((uint32_t)(tile.m0 + wm * 128 + g * 4) * (uint32_t)args.ldc + (uint32_t)(tile.grp * N + col)) * 2u;
-        auto store_all = [&](auto with_bias, half4 bias4) {
+        auto store_all = [&](auto mode, half4 bias4) {     // mode 0: product, 1: + bias, 2: gelu(+ bias)
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
 #pragma unroll
@@ -460,7 +462,9 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
               half4 o;
 #pragma unroll
               for (int j = 0; j < 4; ++j) o[j] = f2h(acc[i][j][r]);
-              if (decltype(with_bias)::value) o = o + bias4;   // half add on the rounded product, as the reference's next kernel does
+              // half add on the rounded product, as the reference's next kernel does (mode 2: and its GELU)
+              if (decltype(mode)::value == 2) o = bias_gelu_half<half4, 4>(o, bias4);
+              else if (decltype(mode)::value == 1) o = o + bias4;
               __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, o), rc, voff, 0, 2 /* nt */);
               voff += row_bytes;
             }
@@ -468,9 +472,12 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
           }
         };
         if (args.bias[tile.grp] != nullptr)
-          store_all(std::true_type{}, *reinterpret_cast<const half4*>((const _Float16*)args.bias[tile.grp] + col));
+          if (args.gelu)
+            store_all(std::integral_constant<int, 2>{}, *reinterpret_cast<const half4*>((const _Float16*)args.bias[tile.grp] + col));
+          else
+            store_all(std::integral_constant<int, 1>{}, *reinterpret_cast<const half4*>((const _Float16*)args.bias[tile.grp] + col));
         else
-          store_all(std::false_type{}, half4{});
+          store_all(std::integral_constant<int, 0>{}, half4{});
       }
     }
     if (!has_next) break;
@@ -810,7 +817,10 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * 32 * WB + i * 32 + 8 * (r >> 2) + 4 * kb + (r & 3);
-        if (row < rows) C[(size_t)row * args.ldc] = acc[i][j][r] + bias;
+        if (row < rows) {
+          const float x = acc[i][j][r] + bias;
+          C[(size_t)row * args.ldc] = args.gelu ? x * gelu_cdf(x, x * x * x) : x;
+        }
       }
   }
 }
@@ -925,10 +935,6 @@ bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int 
   return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && (long)n * groups >= 2L * k;
 }
 
-bool gemm_fuses_bias_gelu(DType t, int m_bound, int ldc, int n, int k, int groups, bool b_transposed) {
-  return b_transposed && gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups);
-}
-
 void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, const SeqStartJob* seq) {
   if (jobs.count == 0 && seq == nullptr) return;
   TransposeArgs a;
@@ -966,7 +972,7 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.n = n;
   a.k = k;
   a.groups = g.groups;
-  a.gelu = g.gelu ? 1 : 0;        // only where gemm_fuses_bias_gelu() holds; the other kernels ignore it
+  a.gelu = g.gelu ? 1 : 0;
   if (t == DType::F16) {
     if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
       launch_f16_persistent(a, stream, g.b_transposed);

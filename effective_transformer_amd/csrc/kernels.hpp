@@ -87,8 +87,8 @@ struct GemmGroups {
   // true: B[g] holds the transpose, [n][k] row-major (see launch_transpose_weights); only where
   // gemm_takes_transposed_b() says so
   bool b_transposed = false;
-  // C = gelu(A.B + bias) (bias + GELU as in launch_bias_gelu, same rounding points); only where
-  // gemm_fuses_bias_gelu() says so, bias[g] must be set
+  // C = gelu(A.B + bias): bias + GELU as in launch_bias_gelu, same rounding points, applied to each tile on its way
+  // out; bias[g] must be set
   bool gelu = false;
 };
 bool gemm_supported(DType t, int n, int k, int groups);
@@ -97,8 +97,6 @@ bool gemm_supported(DType t, int n, int k, int groups);
 bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
 // ... and where the encoder layer found the extra copy worth its time (measured inside the layer, not in isolation).
 bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
-// True when launch_gemm would run a kernel whose epilogue can apply bias + GELU (the large-M kernel on transposed B).
-bool gemm_fuses_bias_gelu(DType t, int m_bound, int ldc, int n, int k, int groups, bool b_transposed);
 // dst[j] ([n][k], row-major) = transpose of src[j] ([k][n], row-major), fp16, one launch for all jobs.
 struct TransposeJobs {
   static constexpr int kMax = 6;

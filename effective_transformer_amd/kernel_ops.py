@@ -99,13 +99,14 @@ def attention(q, k, v, layout: int, packed_ld: int, attr_mask, valid_word_num, B
 
 
 def gemm(a, b, bias=None, m: Optional[int] = None, m_dev: Optional[torch.Tensor] = None,
-         out: Optional[torch.Tensor] = None):
+         out: Optional[torch.Tensor] = None, gelu: bool = False):
+    """a [m, k] . b [k, n] (+ bias); gelu=True applies bias + GELU to the product on its way out."""
     rows, k = a.shape
     n = b.shape[1]
     if out is None:
         out = torch.zeros(rows, n, dtype=a.dtype, device=a.device)
-    _call("et_gemm", a.device, _dtype_code(a.dtype), _p(a), _p(b), _p(out), _p(bias), rows if m is None else m, n, k,
-          _p(m_dev), _stream())
+    _call("et_gemm_bias_gelu" if gelu else "et_gemm", a.device, _dtype_code(a.dtype), _p(a), _p(b), _p(out), _p(bias),
+          rows if m is None else m, n, k, _p(m_dev), _stream())
     return out
 
 

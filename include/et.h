@@ -229,6 +229,12 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
 et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias,
                   int m, int n, int k, const int32_t* m_dev, void* stream);
 
+/* C[m,n] = gelu(A[m,k] . B[k,n] + bias[n]): et_gemm followed by et_add_bias_act in one launch, same arithmetic and
+ * rounding points as the two calls in a row (reference: the cublasGemmEx call and the add_bias_act launch behind it,
+ * tf_op/bert_transformer_op.cu.cc:215-227, cuda/cuda_kernels.cu:29-51, 88-150).  bias is required. */
+et_status et_gemm_bias_gelu(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias,
+                            int m, int n, int k, const int32_t* m_dev, void* stream);
+
 /* dst[n][k] = transpose of src[k][n] (both row-major), fp16 only.  No counterpart in the reference, which hands the
  * TF dense kernels [in,out] to cuBLAS as they are; et_layer does this internally for its large-M GEMMs. */
 et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void* dst, int k, int n, void* stream);

@@ -345,6 +345,25 @@ def test_gemm_bt(k, m, n, k_):
     assert np.array_equal(got2[:m - 301], got[:m - 301]) and np.all(got2[m - 301:] == 0)
 
 
+# every GEMM kernel behind et_gemm: fp32 128x128 and 64x64 tiles, fp16 64- and 128-row tiles, fp16 persistent
+@pytest.mark.parametrize("dtype,m,n,k_", [("fp32", 700, 256, 64), ("fp32", 3000, 3072, 96), ("fp16", 300, 512, 64),
+                                           ("fp16", 5000, 3072, 96), ("fp16", 11000, 1032, 160)])
+def test_gemm_bias_gelu_equals_the_two_passes(k, dtype, m, n, k_):
+    print("gemm_bias_gelu", dtype, m, n, k_, flush=True)
+    rng = np.random.RandomState(m + n + k_ + 2)
+    a = o.rnd(rng.randn(m, k_), dtype)
+    b = o.rnd(0.05 * rng.randn(k_, n), dtype)
+    bias = o.rnd(rng.randn(n), dtype)
+    two = k.add_bias_act(k.gemm(dev(a), dev(b)), dev(bias)).cpu().numpy()
+    one = k.gemm(dev(a), dev(b), bias=dev(bias), gelu=True).cpu().numpy()
+    assert np.array_equal(one, two) and one.tobytes() == two.tobytes()       # same rounding points, bit for bit
+    md = torch.tensor([m - 77], dtype=torch.int32, device="cuda")
+    part = k.gemm(dev(a), dev(b), bias=dev(bias), m_dev=md, gelu=True).cpu().numpy()
+    assert np.array_equal(part[:m - 77], one[:m - 77]) and np.all(part[m - 77:] == 0)
+    with pytest.raises(Exception, match="null bias"):
+        k.gemm(dev(a), dev(b), gelu=True)
+
+
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (5000, 3072, 768)])
 def test_gemm_bt_bias_gelu_equals_the_two_passes(k, m, n, k_):
     print("gemm_bt_bias_gelu", m, n, k_, flush=True)
