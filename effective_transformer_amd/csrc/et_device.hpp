@@ -119,8 +119,8 @@ __device__ __forceinline__ _Float16 f2h(float f) { return (_Float16)f; }   // v_
 // 0.5*(1+tanh(u)) is evaluated as 1/(1+exp(-2u)), which is the same function without the cancellation of 1+tanh for
 // negative u.
 __device__ __forceinline__ float gelu_cdf(float x, float x3) {
-  const float u = 0.7978845608028654f * (x + 0.044715f * x3);
-  const float e = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);      // exp(-2u) = 2^(-2u*log2(e))
+  // exp(-2u) = 2^(-2u*log2(e)) with u = 0.7978845608028654 * (x + 0.044715 * x3): both factors in one constant
+  const float e = __builtin_amdgcn_exp2f((x + 0.044715f * x3) * (-2.8853900817779268f * 0.7978845608028654f));
   return __builtin_amdgcn_rcpf(1.0f + e);
 }
 // fp16 rounding points of the reference: __hadd2 for the bias, two __hmul2 for the cube, the CDF in float rounded to
