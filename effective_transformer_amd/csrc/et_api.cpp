@@ -99,16 +99,21 @@ LayerWs layer_ws(et_dtype dtype, int B, int S, int heads, int d) {
   return w;
 }
 
-// Guard that makes the handle's device current and serialises calls on the handle.
-struct Scope {
-  std::lock_guard<std::mutex> lock;
-  explicit Scope(et_handle h) : lock(h->mu) {}
+// First statement of every entry point that takes a handle: rejects a null handle, takes the handle's lock (calls on
+// one handle are serialised, and the handle's message slot is only written under it) and makes the handle's device
+// current for the calling thread.
+struct Entry {
+  std::unique_lock<std::mutex> lock;
+  et_status status = ET_OK;
+  explicit Entry(et_handle h) {
+    if (!h) {
+      status = fail(nullptr, ET_INVALID_ARGUMENT, "null handle");
+      return;
+    }
+    lock = std::unique_lock<std::mutex>(h->mu);
+    status = check_hip(h, hipSetDevice(h->device), "hipSetDevice", __FILE__, __LINE__);
+  }
 };
-
-et_status enter(et_handle h) {
-  if (!h) return fail(nullptr, ET_INVALID_ARGUMENT, "null handle");
-  return check_hip(h, hipSetDevice(h->device), "hipSetDevice", __FILE__, __LINE__);
-}
 
 et_status dims_ok(et_handle h, int B, int S, int heads, int d) {
   ET_REQUIRE(h, B >= 1 && S >= 1 && heads >= 1 && d >= 1, "batch_size, seq_len, head_num, size_per_head must be >= 1");
@@ -186,9 +191,9 @@ et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const i
                    int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx, int batch_size, int seq_len,
                    int head_num, int size_per_head, void* workspace, size_t workspace_bytes, void* stream,
                    int32_t* valid_word_num_host) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && mask && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
@@ -218,9 +223,9 @@ et_status et_embedding_input(et_handle h, et_dtype dtype, const et_embedding_wei
                              int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx, int batch_size,
                              int seq_len, int head_num, int size_per_head, void* workspace, size_t workspace_bytes,
                              void* stream, int32_t* valid_word_num_host) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, emb != nullptr, "null embeddings");
@@ -259,9 +264,9 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
                    const int32_t* batch_idx, const int32_t* word_idx, void* out, int batch_size, int from_seq_len,
                    int to_seq_len, int head_num, int size_per_head, int valid_word_num_hint, void* workspace,
                    size_t workspace_bytes, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, from_seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, from_seq_len == to_seq_len, "only support from_seq_len == to_seq_len");
@@ -367,9 +372,8 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
 et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* valid_word_num_dev,
                     const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor, int batch_size, int seq_len,
                     int head_num, int size_per_head, void* stream) {
-  et_status s = enter(h);
-  if (s != ET_OK) return s;
-  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  if (head_num < 1 || size_per_head < 1 || (long)head_num * size_per_head >= (1L << 30))
+    return fail(nullptr, ET_INVALID_ARGUMENT, "head_num, size_per_head must be >= 1");
   return et_restore(h, dtype, to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size, seq_len,
                     head_num * size_per_head, stream);
 }
@@ -377,9 +381,9 @@ et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const 
 et_status et_first_token(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* valid_word_num_dev,
                          const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor, int batch_size,
                          int seq_len, int hidden_dim, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
@@ -392,9 +396,9 @@ et_status et_first_token(et_handle h, et_dtype dtype, const void* from_tensor, c
 
 et_status et_exclusive_scan(et_handle h, int32_t* d_out, const int32_t* d_in, int length, void* workspace,
                             size_t workspace_bytes, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, d_out && d_in, "null tensor pointer");
   ET_REQUIRE(h, length >= 1 && length < (1 << 30), "length out of range");
   ET_REQUIRE(h, workspace != nullptr, "null workspace");
@@ -407,9 +411,9 @@ et_status et_exclusive_scan(et_handle h, int32_t* d_out, const int32_t* d_in, in
 et_status et_compress(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask,
                       const int32_t* prefix_sum, void* to_tensor, int32_t* batch_idx, int32_t* word_idx,
                       int batch_size, int seq_len, int hidden_dim, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && mask && prefix_sum && to_tensor && batch_idx && word_idx, "null tensor pointer");
@@ -427,9 +431,9 @@ et_status et_compress(et_handle h, et_dtype dtype, const void* from_tensor, cons
 et_status et_restore(et_handle h, et_dtype dtype, void* to_tensor, const void* from_tensor, const int32_t* batch_idx,
                      const int32_t* word_idx, const int32_t* valid_word_num_dev, int batch_size, int seq_len,
                      int hidden_dim, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
@@ -444,9 +448,9 @@ et_status et_restore(et_handle h, et_dtype dtype, void* to_tensor, const void* f
 
 et_status et_add_bias_act(et_handle h, et_dtype dtype, void* out, const void* bias, int m, int n,
                           const int32_t* m_dev, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   ET_REQUIRE(h, out && bias, "null tensor pointer");
   ET_REQUIRE(h, m >= 0 && n >= 1, "bad dimensions");
@@ -459,9 +463,9 @@ et_status et_add_bias_act(et_handle h, et_dtype dtype, void* out, const void* bi
 et_status et_add_bias_input_layernorm(et_handle h, et_dtype dtype, void* out, const void* input, const void* bias,
                                       const void* gamma, const void* beta, int m, int n, const int32_t* m_dev,
                                       void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   ET_REQUIRE(h, out && input && bias && gamma && beta, "null tensor pointer");
   ET_REQUIRE(h, m >= 0 && n >= 1, "bad dimensions");
@@ -477,9 +481,9 @@ et_status et_add_qkv_bias_padding(et_handle h, et_dtype dtype, const void* Q, co
                                   void* v_buf, const int32_t* valid_word_num_dev, int batch_size, int seq_len,
                                   int head_num, int size_per_head, const int32_t* batch_idx, const int32_t* word_idx,
                                   void* workspace, size_t workspace_bytes, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, Q && K && V && bias_Q && bias_K && bias_V && q_buf && k_buf && v_buf && valid_word_num_dev &&
@@ -499,9 +503,9 @@ et_status et_add_qkv_bias_padding(et_handle h, et_dtype dtype, const void* Q, co
 
 et_status et_softmax(et_handle h, et_dtype dtype, void* qk_buf, const void* attr_mask, int batch_size, int head_num,
                      int seq_len, float scaler, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, 1)) != ET_OK) return s;
   ET_REQUIRE(h, qk_buf && attr_mask, "null tensor pointer");
@@ -513,9 +517,9 @@ et_status et_softmax(et_handle h, et_dtype dtype, void* qk_buf, const void* attr
 et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, void* dst,
                                   const int32_t* valid_word_num_dev, int batch_size, int seq_len, int head_num,
                                   int size_per_head, const int32_t* batch_idx, const int32_t* word_idx, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, src && dst && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
@@ -530,9 +534,9 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
                        int packed_ld, const void* attr_mask, void* dst, const int32_t* valid_word_num_dev,
                        int batch_size, int seq_len, int head_num, int size_per_head, const int32_t* batch_idx,
                        const int32_t* word_idx, void* workspace, size_t workspace_bytes, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, q && k && v && attr_mask && dst && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
@@ -556,9 +560,9 @@ namespace {
 
 et_status gemm_impl(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias, int m, int n,
                     int k, const int32_t* m_dev, void* stream, bool gelu, const char* what) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   ET_REQUIRE(h, A && B && C, "null tensor pointer");
   ET_REQUIRE(h, !gelu || bias, "null bias");
@@ -590,9 +594,9 @@ et_status et_gemm_bias_gelu(et_handle h, et_dtype dtype, const void* A, const vo
 }
 
 et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void* dst, int k, int n, void* stream) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype == ET_FP16, "dtype must be ET_FP16");
   ET_REQUIRE(h, src && dst && src != dst, "null or aliased tensor pointer");
   ET_REQUIRE(h, k >= 1 && n >= 1 && k % 8 == 0 && n % 8 == 0, "k and n must be positive multiples of 8");
@@ -606,9 +610,9 @@ namespace {
 
 et_status gemm_bt_impl(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias, int m, int n,
                        int k, const int32_t* m_dev, void* stream, bool gelu, const char* what) {
-  et_status s = enter(h);
+  Entry entry(h);
+  et_status s = entry.status;
   if (s != ET_OK) return s;
-  Scope scope(h);
   ET_REQUIRE(h, dtype == ET_FP16, "dtype must be ET_FP16");
   ET_REQUIRE(h, A && Bt && C, "null tensor pointer");
   ET_REQUIRE(h, !gelu || bias, "null bias");

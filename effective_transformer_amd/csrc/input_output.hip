@@ -102,7 +102,9 @@ __global__ __launch_bounds__(kScanThreads) void scan_index_kernel(const int32_t*
     if (idx < end) {
       if (prefix_out) prefix_out[idx] = excl;
       if (seq_len > 0) {
-        if (v > 0) {                       // the reference tests mask > 0.5 (cuda_kernels.cu:292)
+        // the reference tests mask > 0.5 (cuda_kernels.cu:292); a mask with entries above 1 would push the prefix sum
+        // past the arrays, which have n slots
+        if (v > 0 && excl < n) {
           const int b = idx / seq_len;
           batch_idx[excl] = b;
           word_idx[excl] = idx - b * seq_len;
@@ -291,7 +293,7 @@ void launch_scan_index(const int32_t* in, int length, int32_t* prefix_out, int32
                        int32_t* valid_word_num, int seq_len, int32_t* scratch, hipStream_t stream) {
   const int tile = scan_tile_for(length);
   const int tiles = (length + tile - 1) / tile;
-  // up to 256 tiles every workgroup re-adds the elements in front of its tile itself (at most 1 MB of L2 reads);
+  // up to 128 tiles every workgroup re-adds the elements in front of its tile itself (at most 508 KB of L2 reads);
   // beyond that a first kernel leaves the tile totals in the scratch
   const bool direct = tiles <= 128 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
   if (!direct) scan_tile_sums_kernel<<<tiles, kScanThreads, 0, stream>>>(in, length, tile, scratch);

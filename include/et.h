@@ -48,8 +48,9 @@ typedef struct et_context* et_handle;
  * (cublasCreate at tf_op/bert_transformer_op.cc:171).  `device` is a HIP device ordinal. */
 et_status et_create(et_handle* out, int device);
 et_status et_destroy(et_handle h);
-/* Message of the last failing call on `h` (or of the last failing et_create on this thread
- * when h is NULL).  Never NULL. */
+/* Message of the last failing call on `h` (or, when h is NULL, of the last call on this thread that failed without a
+ * handle: et_create, a NULL handle argument).  Never NULL.  The handle's message is rewritten by the next failing call
+ * on it: with several threads on one handle, read it before another thread's call can fail. */
 const char* et_last_error(et_handle h);
 const char* et_status_string(et_status s);
 /* 1 when the library was built for the architecture of `device` and a kernel runs there. */
