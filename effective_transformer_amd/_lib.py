@@ -28,6 +28,12 @@ class LayerWeights(C.Structure):
     _fields_ = [(name, C.c_void_p) for name in WEIGHT_FIELDS]
 
 
+class LayerPrepared(C.Structure):
+    _fields_ = [("attr_kernel_Q_t", C.c_void_p), ("attr_kernel_K_t", C.c_void_p), ("attr_kernel_V_t", C.c_void_p),
+                ("attr_output_kernel_t", C.c_void_p), ("inter_kernel_t", C.c_void_p), ("output_kernel_t", C.c_void_p),
+                ("seq_start", C.c_void_p)]
+
+
 class EmbeddingWeights(C.Structure):
     _fields_ = [("word_embeddings", C.c_void_p), ("token_type_embeddings", C.c_void_p),
                 ("position_embeddings", C.c_void_p), ("layernorm_gamma", C.c_void_p), ("layernorm_beta", C.c_void_p),
@@ -57,6 +63,9 @@ SIGNATURES = {
                                 _vp, _sz, _vp, _ip]),
     "et_layer": (_i, [_vp, _i, C.POINTER(LayerWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                       _vp, _sz, _vp]),
+    "et_sequence_starts": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "et_layer_with_prepared": (_i, [_vp, _i, C.POINTER(LayerWeights), C.POINTER(LayerPrepared), _vp, _vp, _vp, _vp, _vp,
+                                    _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "et_first_token": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "et_output": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "et_exclusive_scan": (_i, [_vp, _vp, _vp, _i, _vp, _sz, _vp]),

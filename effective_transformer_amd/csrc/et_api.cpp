@@ -264,6 +264,28 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
                    const int32_t* batch_idx, const int32_t* word_idx, void* out, int batch_size, int from_seq_len,
                    int to_seq_len, int head_num, int size_per_head, int valid_word_num_hint, void* workspace,
                    size_t workspace_bytes, void* stream) {
+  return et_layer_with_prepared(h, dtype, w, nullptr, from_tensor, to_tensor, attr_mask, valid_word_num_dev, batch_idx,
+                                word_idx, out, batch_size, from_seq_len, to_seq_len, head_num, size_per_head,
+                                valid_word_num_hint, workspace, workspace_bytes, stream);
+}
+
+et_status et_sequence_starts(et_handle h, const int32_t* batch_idx, const int32_t* valid_word_num_dev, int batch_size,
+                             int seq_len, int32_t* seq_start, void* stream) {
+  Entry entry(h);
+  et_status s = entry.status;
+  if (s != ET_OK) return s;
+  if ((s = dims_ok(h, batch_size, seq_len, 1, 1)) != ET_OK) return s;
+  ET_REQUIRE(h, batch_idx && valid_word_num_dev && seq_start, "null tensor pointer");
+  et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, seq_start, (hipStream_t)stream);
+  return check_launch(h, "sequence starts");
+}
+
+et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_weights* w, const et_layer_prepared* prep,
+                                 const void* from_tensor, const void* to_tensor, const void* attr_mask,
+                                 const int32_t* valid_word_num_dev, const int32_t* batch_idx, const int32_t* word_idx,
+                                 void* out, int batch_size, int from_seq_len, int to_seq_len, int head_num,
+                                 int size_per_head, int valid_word_num_hint, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
   Entry entry(h);
   et_status s = entry.status;
   if (s != ET_OK) return s;
@@ -305,29 +327,45 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
   void* inter = base + ws.inter;
   int32_t* seq_start = (int32_t*)(base + ws.seq);
 
-  // The large-M fp16 GEMM reads k-contiguous weights with fewer LDS instructions; for the wide projections that is
-  // worth a transposed copy in the workspace per call (the caller's weights stay as they are).
-  const bool t_qkv = et::gemm_prefers_transposed_b(dt, rows, 3 * H, H, H, 3);
-  const bool t_o = et::gemm_prefers_transposed_b(dt, rows, H, H, H, 1);
-  const bool t_up = et::gemm_prefers_transposed_b(dt, rows, F, F, H, 1);
-  const bool t_down = et::gemm_prefers_transposed_b(dt, rows, H, H, F, 1);
+  // The large-M fp16 GEMM reads k-contiguous weights with fewer LDS instructions.  Where the caller prepared such
+  // copies they are used wherever that kernel runs; otherwise the wide projections get a transposed copy in the
+  // workspace on every call (the caller's weights stay as they are).
+  static const et_layer_prepared kNoPrep = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  const et_layer_prepared& pp = prep ? *prep : kNoPrep;
+  ET_REQUIRE(h, (pp.attr_kernel_Q_t != nullptr) == (pp.attr_kernel_K_t != nullptr) &&
+                    (pp.attr_kernel_Q_t != nullptr) == (pp.attr_kernel_V_t != nullptr),
+             "prepared Q, K and V kernels go together");
+  const bool can_qkv = et::gemm_takes_transposed_b(dt, rows, 3 * H, H, H, 3);
+  const bool can_o = et::gemm_takes_transposed_b(dt, rows, H, H, H, 1);
+  const bool can_up = et::gemm_takes_transposed_b(dt, rows, F, F, H, 1);
+  const bool can_down = et::gemm_takes_transposed_b(dt, rows, H, H, F, 1);
+  const bool t_qkv = can_qkv && (pp.attr_kernel_Q_t || et::gemm_prefers_transposed_b(dt, rows, 3 * H, H, H, 3));
+  const bool t_o = can_o && (pp.attr_output_kernel_t || et::gemm_prefers_transposed_b(dt, rows, H, H, H, 1));
+  const bool t_up = can_up && (pp.inter_kernel_t || et::gemm_prefers_transposed_b(dt, rows, F, F, H, 1));
+  const bool t_down = can_down && (pp.output_kernel_t || et::gemm_prefers_transposed_b(dt, rows, H, H, F, 1));
   char* wt = base + ws.wt;
   const size_t HH = (size_t)H * H * e;
-  void* wt_q = wt; void* wt_k = wt + HH; void* wt_v = wt + 2 * HH; void* wt_o = wt + 3 * HH;
-  void* wt_up = wt + 4 * HH; void* wt_down = wt + 8 * HH;
+  const void* wt_q = wt; const void* wt_k = wt + HH; const void* wt_v = wt + 2 * HH; const void* wt_o = wt + 3 * HH;
+  const void* wt_up = wt + 4 * HH; const void* wt_down = wt + 8 * HH;
   {
     et::TransposeJobs jobs;
-    if (t_qkv) {
-      jobs.add(w->attr_kernel_Q, wt_q, H, H);
-      jobs.add(w->attr_kernel_K, wt_k, H, H);
-      jobs.add(w->attr_kernel_V, wt_v, H, H);
+    if (t_qkv && pp.attr_kernel_Q_t) {
+      wt_q = pp.attr_kernel_Q_t; wt_k = pp.attr_kernel_K_t; wt_v = pp.attr_kernel_V_t;
+    } else if (t_qkv) {
+      jobs.add(w->attr_kernel_Q, wt, H, H);
+      jobs.add(w->attr_kernel_K, wt + HH, H, H);
+      jobs.add(w->attr_kernel_V, wt + 2 * HH, H, H);
     }
-    if (t_o) jobs.add(w->attr_output_kernel, wt_o, H, H);
-    if (t_up) jobs.add(w->inter_kernel, wt_up, H, F);
-    if (t_down) jobs.add(w->output_kernel, wt_down, F, H);
-    // one launch builds the sequence start table and the transposed copies
+    if (t_o && pp.attr_output_kernel_t) wt_o = pp.attr_output_kernel_t;
+    else if (t_o) jobs.add(w->attr_output_kernel, wt + 3 * HH, H, H);
+    if (t_up && pp.inter_kernel_t) wt_up = pp.inter_kernel_t;
+    else if (t_up) jobs.add(w->inter_kernel, wt + 4 * HH, H, F);
+    if (t_down && pp.output_kernel_t) wt_down = pp.output_kernel_t;
+    else if (t_down) jobs.add(w->output_kernel, wt + 8 * HH, F, H);
+    // one launch builds the sequence start table and the transposed copies; none when the caller prepared both
     const et::SeqStartJob seq{batch_idx, T, rows, B, seq_start};
-    et::launch_transpose_weights(jobs, st, &seq);
+    if (pp.seq_start) seq_start = const_cast<int32_t*>(pp.seq_start);
+    et::launch_transpose_weights(jobs, st, pp.seq_start ? nullptr : &seq);
   }
   // Q = from.Wq + bq, K = to.Wk + bk, V = to.Wv + bv into one [T,3H] buffer (bert_transformer_op.cu.cc:105-156)
   et::GemmGroups g3;

@@ -191,6 +191,35 @@ class LayerWeights:
                      "output_layernorm_gamma", "output_layernorm_beta"):
             setattr(s, name, self.t[name].data_ptr())
         self.struct = s
+        self.prepared: Optional[_lib.LayerPrepared] = None
+        self._prepared_tensors: List[torch.Tensor] = []
+
+    def prepare(self, every_kernel: bool = True) -> "LayerWeights":
+        """For weights that stay as they are: k-contiguous ([out,in]) copies of the dense kernels, made once, which the
+        layer op then uses for its large-M GEMMs instead of transposing on every call (fp16 only; a no-op for fp32).
+        every_kernel=False: only the kernels of the wide projections (Q, K, V, FFN up), the ones the layer op would
+        transpose by itself."""
+        if self.t["attr_kernel_q"].dtype != torch.float16:
+            return self
+        lib = _lib.load()
+        dev = self.t["attr_kernel_q"].device
+        h = handle(dev)
+        prep = _lib.LayerPrepared()
+        names = [("attr_kernel_q", "attr_kernel_Q_t"), ("attr_kernel_k", "attr_kernel_K_t"),
+                 ("attr_kernel_v", "attr_kernel_V_t"), ("inter_kernel", "inter_kernel_t")]
+        if every_kernel:
+            names += [("attr_output_kernel", "attr_output_kernel_t"), ("output_kernel", "output_kernel_t")]
+        self._prepared_tensors = []
+        with torch.cuda.device(dev):
+            for src_name, field in names:
+                src = self.t[src_name]
+                k, n = src.shape
+                dst = torch.empty(n, k, dtype=src.dtype, device=dev)
+                _lib.check(lib.et_transpose_weight(h, _lib.ET_FP16, _p(src), _p(dst), k, n, _stream()), h)
+                self._prepared_tensors.append(dst)
+                setattr(prep, field, dst.data_ptr())
+        self.prepared = prep
+        return self
 
     @classmethod
     def from_slots(cls, device, dtype, slots: Sequence):
@@ -212,9 +241,11 @@ def effective_transformer(from_tensor: torch.Tensor, to_tensor: torch.Tensor, at
                           valid_word_num: torch.Tensor, batch_idx: torch.Tensor, word_idx: torch.Tensor,
                           weights: LayerWeights, batch_size: int, from_seq_len: int, to_seq_len: int, head_num: int,
                           size_per_head: int, valid_word_num_hint: int = -1,
-                          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          out: Optional[torch.Tensor] = None, seq_start: Optional[torch.Tensor] = None) -> torch.Tensor:
     """EffectiveTransformer layer op (tf_op/bert_transformer_op.cc:44-77, 180-221).  Output has
-    the shape of from_tensor; rows beyond the valid-token count are left as allocated."""
+    the shape of from_tensor; rows beyond the valid-token count are left as allocated.
+    seq_start: the table of `sequence_starts` for this batch (saves building it in every layer); weights that were
+    `prepare()`d bring their transposed kernels along."""
     lib = _lib.load()
     _require_cuda(from_tensor, to_tensor, attr_mask, valid_word_num, batch_idx, word_idx)
     B = from_tensor.shape[0]
@@ -227,10 +258,31 @@ def effective_transformer(from_tensor: torch.Tensor, to_tensor: torch.Tensor, at
     nbytes = lib.et_layer_workspace_bytes(code, B, from_seq_len, head_num, size_per_head)
     ws = _workspace(dev, "layer", nbytes)
     h = handle(dev)
-    st = lib.et_layer(h, code, C.byref(weights.struct), _p(from_tensor), _p(to_tensor), _p(attr_mask),
-                      _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B, from_seq_len, to_seq_len, head_num,
-                      size_per_head, valid_word_num_hint, _p(ws), ws.numel(), _stream())
+    if weights.prepared is None and seq_start is None:
+        st = lib.et_layer(h, code, C.byref(weights.struct), _p(from_tensor), _p(to_tensor), _p(attr_mask),
+                          _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B, from_seq_len, to_seq_len,
+                          head_num, size_per_head, valid_word_num_hint, _p(ws), ws.numel(), _stream())
+    else:
+        prep = weights.prepared if weights.prepared is not None else _lib.LayerPrepared()
+        prep.seq_start = seq_start.data_ptr() if seq_start is not None else None
+        st = lib.et_layer_with_prepared(h, code, C.byref(weights.struct), C.byref(prep), _p(from_tensor), _p(to_tensor),
+                                        _p(attr_mask), _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B,
+                                        from_seq_len, to_seq_len, head_num, size_per_head, valid_word_num_hint, _p(ws),
+                                        ws.numel(), _stream())
     _lib.check(st, h)
+    return out
+
+
+def sequence_starts(valid_word_num: torch.Tensor, batch_idx: torch.Tensor, batch_size: int, seq_len: int,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """int32[batch_size + 1]: first packed row of every sequence (entry batch_size = valid-token count), the table
+    the attention kernel walks; one per batch serves all layers."""
+    lib = _lib.load()
+    _require_cuda(valid_word_num, batch_idx)
+    if out is None:
+        out = torch.empty(batch_size + 1, dtype=torch.int32, device=batch_idx.device)
+    h = handle(batch_idx.device)
+    _lib.check(lib.et_sequence_starts(h, _p(batch_idx), _p(valid_word_num), batch_size, seq_len, _p(out), _stream()), h)
     return out
 
 
@@ -273,7 +325,9 @@ class EffectiveTransformerEncoder:
     them into op attributes at graph build, python/effective_transformer/__init__.py:48-76)."""
 
     def __init__(self, num_layers: int, head_num: int, size_per_head: int, weights_value: Sequence, dtype: torch.dtype,
-                 device="cuda"):
+                 device="cuda", prepare: bool = True):
+        """prepare: the weights are constants of this object, so the k-contiguous copies the large-M GEMMs want are
+        made here once (fp16) instead of in every layer call."""
         if len(weights_value) != 16 * num_layers:
             raise ValueError("expected %d weight tensors, got %d" % (16 * num_layers, len(weights_value)))
         self.device = torch.device(device)
@@ -283,7 +337,10 @@ class EffectiveTransformerEncoder:
         self.head_num, self.size_per_head, self.num_layers = head_num, size_per_head, num_layers
         self.layers: List[LayerWeights] = [
             LayerWeights.from_slots(self.device, dtype, weights_value[16 * l:16 * l + 16]) for l in range(num_layers)]
-        self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor]] = {}
+        if prepare:
+            for w in self.layers:
+                w.prepare()
+        self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
 
     @classmethod
     def from_checkpoint(cls, path: str, head_num: int, size_per_head: int, dtype: torch.dtype, device="cuda",
@@ -322,12 +379,13 @@ class EffectiveTransformerEncoder:
         key = tuple(x.shape)
         bufs = self._bufs.get(key)
         if bufs is None:
-            bufs = (torch.empty_like(x), torch.empty_like(x))
+            bufs = (torch.empty_like(x), torch.empty_like(x), torch.empty(B + 1, dtype=torch.int32, device=x.device))
             self._bufs[key] = bufs
+        starts = sequence_starts(vwn, bidx, B, S, out=bufs[2])       # one table for all layers of the batch
         for l, w in enumerate(self.layers):
             out = bufs[l & 1]
             effective_transformer(x, x, attention_mask, vwn, bidx, widx, w, B, S, S, hn, d, valid_word_num_hint=T,
-                                  out=out)
+                                  out=out, seq_start=starts)
             x = out
         return effective_transformer_output(x, vwn, bidx, widx, B, S, S, hn, d)
 

@@ -113,6 +113,38 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
                    void* out, int batch_size, int from_seq_len, int to_seq_len, int head_num, int size_per_head,
                    int valid_word_num_hint, void* workspace, size_t workspace_bytes, void* stream);
 
+/* What a caller that keeps a layer's weights constant can prepare once instead of having et_layer redo it on every
+ * call.  No counterpart in the reference, whose op receives the weights as inputs of every call (tf_op/
+ * bert_transformer_op.cc:44-77) and rebuilds nothing across calls either.  Every member may be NULL.
+ *   *_t: the dense kernel handed over [out,in] (k-contiguous), i.e. et_transpose_weight of the [in,out] tensor, fp16
+ *        only.  Used where et_layer would run its large-M GEMM (it then skips its per-call transposition; Q, K and V
+ *        go together); ignored for batches that run the small-M kernels, which read the [in,out] tensors.
+ *   seq_start: int32[batch_size + 1] from et_sequence_starts for THIS batch (first packed row of every sequence);
+ *        the same table serves every layer of the batch. */
+typedef struct et_layer_prepared {
+  const void* attr_kernel_Q_t;       /* [H,H]  */
+  const void* attr_kernel_K_t;       /* [H,H]  */
+  const void* attr_kernel_V_t;       /* [H,H]  */
+  const void* attr_output_kernel_t;  /* [H,H]  */
+  const void* inter_kernel_t;        /* [4H,H] */
+  const void* output_kernel_t;       /* [H,4H] */
+  const int32_t* seq_start;          /* [B+1]  */
+} et_layer_prepared;
+
+/* seq_start[b] = first packed row of sequence b for b in [0,B), seq_start[B] = T: the table the attention kernel
+ * walks, from the index arrays et_input produced.  No counterpart in the reference (its attention works on padded
+ * buffers). */
+et_status et_sequence_starts(et_handle h, const int32_t* batch_idx, const int32_t* valid_word_num_dev, int batch_size,
+                             int seq_len, int32_t* seq_start, void* stream);
+
+/* et_layer with prepared data (see et_layer_prepared; NULL = et_layer).  Same results, bit for bit. */
+et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_weights* weights,
+                                 const et_layer_prepared* prepared, const void* from_tensor, const void* to_tensor,
+                                 const void* attr_mask, const int32_t* valid_word_num_dev, const int32_t* batch_idx,
+                                 const int32_t* word_idx, void* out, int batch_size, int from_seq_len, int to_seq_len,
+                                 int head_num, int size_per_head, int valid_word_num_hint, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
 /* EffectiveTransformerOutputOpFunctor::Compute, tf_op/bert_transformer_op.cu.cc:339-373
  * (op registered at tf_op/bert_transformer_op.cc:359-380): to_tensor [B,S,H] = 0 at padding,
  * from_tensor row t at (batch_idx[t], word_idx[t]).  batch_idx/word_idx must be those written

@@ -72,8 +72,35 @@ class DeviceBuffer {
 // object owns only its scratch: packed activations, index arrays, workspaces.  Not thread-safe; one object per stream.
 class Encoder {
  public:
-  Encoder(int device, et_dtype dtype, int head_num, int size_per_head, std::vector<et_layer_weights> layers)
-      : handle_(device), dtype_(dtype), heads_(head_num), d_(size_per_head), layers_(std::move(layers)) {}
+  // prepare: the weights stay as they are for the life of this object, so the k-contiguous copies of the dense kernels
+  // that the large-M fp16 GEMMs want are made here once (on the device's default stream, waited for) instead of in
+  // every layer call.
+  Encoder(int device, et_dtype dtype, int head_num, int size_per_head, std::vector<et_layer_weights> layers,
+          bool prepare = true)
+      : handle_(device), dtype_(dtype), heads_(head_num), d_(size_per_head), layers_(std::move(layers)) {
+    prepared_.assign(layers_.size(), et_layer_prepared{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr});
+    if (!prepare || dtype != ET_FP16) return;
+    check_hip(hipSetDevice(device), "hipSetDevice");
+    const size_t H = (size_t)head_num * size_per_head;
+    char* dst = (char*)wt_.reserve(layers_.size() * 12 * H * H * 2);
+    auto transposed = [&](const void* src, int k, int n) {
+      void* out = dst;
+      check(et_transpose_weight(handle_.get(), ET_FP16, src, out, k, n, nullptr), handle_.get());
+      dst += (size_t)k * n * 2;
+      return (const void*)out;
+    };
+    for (size_t l = 0; l < layers_.size(); ++l) {
+      const et_layer_weights& w = layers_[l];
+      et_layer_prepared& p = prepared_[l];
+      p.attr_kernel_Q_t = transposed(w.attr_kernel_Q, (int)H, (int)H);
+      p.attr_kernel_K_t = transposed(w.attr_kernel_K, (int)H, (int)H);
+      p.attr_kernel_V_t = transposed(w.attr_kernel_V, (int)H, (int)H);
+      p.attr_output_kernel_t = transposed(w.attr_output_kernel, (int)H, (int)H);
+      p.inter_kernel_t = transposed(w.inter_kernel, (int)H, (int)(4 * H));
+      p.output_kernel_t = transposed(w.output_kernel, (int)(4 * H), (int)H);
+    }
+    check_hip(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+  }
 
   // from_tensor [B,S,H], mask int32 [B,S], attr_mask [B,S,S] in dtype -> out [B,S,H] (zeros at padding).
   // sync_count: read the valid-token count back once (exact launch sizes, one stream synchronisation, as the reference
@@ -84,8 +111,8 @@ class Encoder {
     const size_t e = dtype_ == ET_FP32 ? 4 : 2;
     const size_t H = (size_t)heads_ * d_, rows = (size_t)batch * seq_len;
     char* act = (char*)act_.reserve(3 * rows * H * e);                 // packed input + two layer outputs
-    int32_t* idx = (int32_t*)idx_.reserve((2 * rows + 1) * sizeof(int32_t));
-    int32_t *batch_idx = idx, *word_idx = idx + rows, *count = idx + 2 * rows;
+    int32_t* idx = (int32_t*)idx_.reserve((2 * rows + 1 + (size_t)batch + 1) * sizeof(int32_t));
+    int32_t *batch_idx = idx, *word_idx = idx + rows, *count = idx + 2 * rows, *starts = idx + 2 * rows + 1;
     const size_t in_ws = et_input_workspace_bytes(batch, seq_len);
     const size_t layer_ws = et_layer_workspace_bytes(dtype_, batch, seq_len, heads_, d_);
     void* ws = ws_.reserve(in_ws > layer_ws ? in_ws : layer_ws);
@@ -93,11 +120,16 @@ class Encoder {
     check(et_input(handle_.get(), dtype_, from_tensor, mask, act, count, batch_idx, word_idx, batch, seq_len, heads_, d_, ws,
                    ws_.capacity(), stream, sync_count ? &host_count : nullptr),
           handle_.get());
+    // one sequence start table serves every layer of the batch
+    check(et_sequence_starts(handle_.get(), batch_idx, count, batch, seq_len, starts, stream), handle_.get());
     const char* x = act;
     for (size_t l = 0; l < layers_.size(); ++l) {
       char* y = act + (1 + (l & 1)) * rows * H * e;
-      check(et_layer(handle_.get(), dtype_, &layers_[l], x, x, attr_mask, count, batch_idx, word_idx, y, batch, seq_len,
-                     seq_len, heads_, d_, sync_count ? host_count : -1, ws, ws_.capacity(), stream),
+      et_layer_prepared prep = prepared_[l];
+      prep.seq_start = starts;
+      check(et_layer_with_prepared(handle_.get(), dtype_, &layers_[l], &prep, x, x, attr_mask, count, batch_idx, word_idx, y,
+                                   batch, seq_len, seq_len, heads_, d_, sync_count ? host_count : -1, ws, ws_.capacity(),
+                                   stream),
             handle_.get());
       x = y;
     }
@@ -111,7 +143,8 @@ class Encoder {
   et_dtype dtype_;
   int heads_, d_;
   std::vector<et_layer_weights> layers_;
-  DeviceBuffer act_, idx_, ws_;
+  std::vector<et_layer_prepared> prepared_;
+  DeviceBuffer act_, idx_, ws_, wt_;
 };
 
 }  // namespace et

@@ -35,15 +35,18 @@ def assert_half_close(got, want, ulps=1.0, frac=0.02, what="", atol=0.0):
         assert (err > 0).mean() <= frac, "%s: %.4f of elements differ" % (what, (err > 0).mean())
 
 
-def run_encoder(w, layers=None, hint=True, dtype=None):
-    """Runs Input -> L x Layer -> Output on the GPU for an oracle workload dict.  Returns
-    (output [B,S,H] numpy, T)."""
+def run_encoder(w, layers=None, hint=True, dtype=None, prepare=True, every_kernel=True):
+    """Runs Input -> L x Layer -> Output on the GPU for an oracle workload dict.  Returns the output [B,S,H] as numpy.
+    prepare=False: plain et_layer calls; every_kernel=False: only the wide projections' kernels pre-transposed."""
     from effective_transformer_amd import ops
     wl = w["wl"]
     dt = TDT[dtype or wl.dtype]
     weights = w["weights"] if layers is None else w["weights"][:16 * layers]
     L = len(weights) // 16
-    enc = ops.EffectiveTransformerEncoder(L, wl.heads, wl.d, weights, dt, "cuda")
+    enc = ops.EffectiveTransformerEncoder(L, wl.heads, wl.d, weights, dt, "cuda", prepare=prepare)
+    if prepare and not every_kernel:
+        for lw in enc.layers:
+            lw.prepare(every_kernel=False)
     x = dev(w["x"], dt)
     mask = dev(w["mask"].astype(np.int32))
     attr = dev(w["attr_mask"], dt)

@@ -92,6 +92,28 @@ def test_full_size_properties_and_subset_oracle(name, nsub, layers):
     assert np.array_equal(run_encoder(wp), full[perm])
 
 
+@pytest.mark.parametrize("name,layers", [("cfg3", 2), ("cfg2", 3), ("cfg4", 1)])
+def test_prepared_weights_and_shared_start_table_change_nothing(name, layers):
+    """et_layer_with_prepared (transposed kernels made once, one sequence start table per batch) against plain et_layer
+    calls: the same bits, with the wide projections' kernels prepared and with all six."""
+    print("prepared", name, flush=True)
+    w = o.make_workload(name)
+    plain = run_encoder(w, layers=layers, prepare=False)
+    assert np.array_equal(run_encoder(w, layers=layers, prepare=True), plain)
+    assert np.array_equal(run_encoder(w, layers=layers, prepare=True, every_kernel=False), plain)
+    assert np.array_equal(run_encoder(w, layers=layers, prepare=True, hint=False), plain)
+
+
+def test_prepared_q_k_v_go_together():
+    from effective_transformer_amd import _lib, ops
+    w = o.make_workload("cfg2")
+    wl = w["wl"]
+    enc = ops.EffectiveTransformerEncoder(1, wl.heads, wl.d, w["weights"][:16], torch.float16, "cuda")
+    enc.layers[0].prepared.attr_kernel_K_t = None
+    with pytest.raises(_lib.EtError, match="go together"):
+        enc(dev(w["x"], torch.float16), dev(w["mask"].astype(np.int32)), dev(w["attr_mask"], torch.float16))
+
+
 def test_empty_batch_of_tokens_and_holes():
     w = o.make_workload("cfg1", random_affine=True)
     wl = w["wl"]
