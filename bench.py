@@ -21,9 +21,9 @@ if ROOT not in sys.path:
 # plain device copy of known size shows in the same run); cfg3 shapes.  (read + write) in bytes.
 MEASURED_TRAFFIC = {
     ("cfg3", "gemm_ffn_up"): (377.2 + 236.7) * (1 << 20),
-    ("cfg3", "gemm_ffn_down"): (327.4 + 59.2) * (1 << 20),
-    ("cfg3", "gemm_qkv"): (241.8 + 177.6) * (1 << 20),
-    ("cfg3", "gemm_attn_out"): (86.2 + 59.3) * (1 << 20),
+    ("cfg3", "gemm_ffn_down"): (328.0 + 59.3) * (1 << 20),
+    ("cfg3", "gemm_qkv"): (241.0 + 177.7) * (1 << 20),
+    ("cfg3", "gemm_attn_out"): (86.0 + 59.3) * (1 << 20),
     ("cfg3", "bias_gelu"): (236.8 + 236.7) * (1 << 20),
     ("cfg3", "bias_residual_layernorm"): (118.4 + 59.2) * (1 << 20),
     ("cfg3", "attention"): (202.2 + 59.2) * (1 << 20),
