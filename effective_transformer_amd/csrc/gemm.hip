@@ -111,7 +111,7 @@ __device__ __forceinline__ void transpose8x8(const uint4v (&raw)[8], half8 (&bop
 }
 
 template <int MI>
-__global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
+__global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f16_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass only needs the stub
   using Tile = HTile<MI>;
   constexpr int BM = Tile::BM, BN = kHBN;
@@ -187,25 +187,25 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
   for (int q = 0; q < kStages; ++q) issue(q);
   wait_vmcnt<Tile::DMA * (kStages - 1)>();
   barrier_only();
-  half8 a_cur[MI], bop_cur[8];
+  // Two operand register sets: a k-step multiplies out of one while it fills the other, and the k loop below is
+  // unrolled by two so that neither set is ever copied.
+  half8 a_reg[2][MI], b_reg[2][8];
   {
     uint4v raw[8];
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint4v*>(smem + Tile::A_BYTES + b_rd + kk * BN * 2);
 #pragma unroll
-    for (int i = 0; i < MI; ++i) a_cur[i] = *reinterpret_cast<const half8*>(smem + a_rd + i * 16 * 64);
-    transpose8x8(raw, bop_cur);
+    for (int i = 0; i < MI; ++i) a_reg[0][i] = *reinterpret_cast<const half8*>(smem + a_rd + i * 16 * 64);
+    transpose8x8(raw, b_reg[0]);
   }
 
-  for (int kt = 0; kt < nk; ++kt) {
+  auto step = [&](int kt, const half8 (&a_cur)[MI], const half8 (&bop_cur)[8], half8 (&a_n)[MI], half8 (&bop_n)[8]) {
     wait_vmcnt<Tile::DMA * (kStages - 2)>();   // k-step kt+1 has landed; kt+2 and kt+3 may still be in flight
     wait_lgkmcnt0();                           // this wavefront's reads of k-step kt's buffer are complete
     barrier_only();
     issue(kt + kStages);                       // into the buffer of k-step kt, free now for every wavefront
-    __builtin_amdgcn_sched_barrier(0);
     const unsigned char* st = smem + ((kt + 1) % kStages) * Tile::STAGE_BYTES;
     uint4v raw[8];
-    half8 a_n[MI], bop_n[8];
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint4v*>(st + Tile::A_BYTES + b_rd + kk * BN * 2);
 #pragma unroll
@@ -216,23 +216,29 @@ __global__ __launch_bounds__(kHThreads) void gemm_f16_kernel(GemmArgs args) {
       for (int j = 0; j < 8; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[i], bop_cur[j], acc[i][j], 0, 0, 0);
     transpose8x8(raw, bop_n);
-    // issue order: LDS reads spread over the first half of the MFMAs, the transposes over the second half
+    // issue order: the MFMAs start right behind the barrier; the LDS reads and this wave's DMA instructions go between
+    // the first of them, the transposes (which wait for the reads) between the rest
+    constexpr int kReads = 8 + MI, kMfma = 8 * MI, kLate = kMfma - kReads;
 #pragma unroll
-    for (int r = 0; r < 8 + MI; ++r) {
+    for (int r = 0; r < kReads; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 LDS read
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
+      if (r < Tile::DMA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 DMA instruction
     }
 #pragma unroll
-    for (int r = 0; r < 32; ++r) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);   // 1 VALU (transpose)
+    for (int r = 0; r < kLate; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, (32 + kLate - 1) / kLate, 0);   // its share of the 32 transposes
     }
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < MI; ++i) a_cur[i] = a_n[i];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) bop_cur[j] = bop_n[j];
+  };
+  int kt = 0;
+#pragma unroll 1
+  for (; kt + 1 < nk; kt += 2) {
+    step(kt, a_reg[0], b_reg[0], a_reg[1], b_reg[1]);
+    step(kt + 1, a_reg[1], b_reg[1], a_reg[0], b_reg[0]);
   }
+  if (kt < nk) step(kt, a_reg[0], b_reg[0], a_reg[1], b_reg[1]);
   wait_vmcnt<0>();        // no DMA may still target this workgroup's LDS when it ends
 
   // epilogue: lane owns rows g*4+r of every 16-row sub-tile and 8 consecutive columns
