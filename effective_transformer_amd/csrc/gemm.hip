@@ -68,14 +68,18 @@ __device__ __forceinline__ int remap_valid_tile(int pid, int valid_tiles) {
 // ------------------------------------------------------------------------------------------
 constexpr int kHThreads = 256;
 constexpr int kHBK = 32;
-constexpr int kHBN = 256;
 constexpr int kStages = 4;
 
-template <int MI>
+// MI: 16-row blocks per wavefront (2 wavefronts along m); NJ: 16-column blocks per wavefront (2 wavefronts along n).
+// NJ = 8 is the 256-column tile; NJ = 4 halves the B bytes a workgroup moves per k-step and doubles the number of
+// workgroups, which is what counts when there are fewer 256-column tiles than CUs.
+template <int MI, int NJ>
 struct HTile {
   static constexpr int BM = 32 * MI;
+  static constexpr int BN = 32 * NJ;
   static constexpr int A_BYTES = BM * kHBK * 2;
-  static constexpr int B_BYTES = kHBK * kHBN * 2;              // 16 KB
+  static constexpr int B_BYTES = kHBK * BN * 2;                // 16 KB / 8 KB
+  static constexpr int B_ROW_CHUNKS = BN / 8;                  // 16-byte chunks per k-row
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int SMEM_BYTES = kStages * STAGE_BYTES;
   static constexpr int A_DMA = A_BYTES / 1024 / 4;             // DMA instructions per wavefront per stage
@@ -95,10 +99,20 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(15 
 __device__ __forceinline__ void barrier_only() { asm volatile("s_barrier" ::: "memory"); }
 
 __device__ __forceinline__ int a_swizzle(int row) { return (row >> 1) & 3; }
+// 128-column B stages: a wavefront reads 8 bytes per lane, 32 lanes per LDS pass, i.e. two groups of 16 lanes whose
+// k-rows are 2 KB apart.  Swapping the two 128-byte halves of every second group of 8 k-rows puts them on different banks.
+template <int NJ>
+__device__ __forceinline__ int b_swizzle(int chunk, int k_row) {
+  return NJ == 8 ? chunk : chunk ^ (((k_row >> 3) & 1) << 3);
+}
 
-__device__ __forceinline__ void transpose8x8(const uint4v (&raw)[8], half8 (&bop)[8]) {
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+// raw[kk]: NJ consecutive columns of k-row kk -> bop[j]: the 8 k values of column j
+template <typename Raw, int NJ>
+__device__ __forceinline__ void transpose8x8(const Raw (&raw)[8], half8 (&bop)[NJ]) {
 #pragma unroll
-  for (int jj = 0; jj < 4; ++jj) {       // dword jj of a raw k-row holds columns 2jj, 2jj+1
+  for (int jj = 0; jj < NJ / 2; ++jj) {       // dword jj of a raw k-row holds columns 2jj, 2jj+1
     uint4v lo, hi;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
@@ -110,11 +124,13 @@ __device__ __forceinline__ void transpose8x8(const uint4v (&raw)[8], half8 (&bop
   }
 }
 
-template <int MI>
+template <int MI, int NJ>
 __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f16_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass only needs the stub
-  using Tile = HTile<MI>;
-  constexpr int BM = Tile::BM, BN = kHBN;
+  using Tile = HTile<MI, NJ>;
+  using Raw = typename std::conditional<NJ == 8, uint4v, uint2v>::type;     // NJ halves of one k-row
+  using HalfN = typename std::conditional<NJ == 8, half8, half4>::type;
+  constexpr int BM = Tile::BM, BN = Tile::BN;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
@@ -153,9 +169,10 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
   }
 #pragma unroll
   for (int j = 0; j < Tile::B_DMA; ++j) {
-    const int q = wave * Tile::B_DMA + j;              // 1 KB slot of the B stage: 2 k-rows x 32 chunks
-    const int kr = q * 2 + (lane >> 5);
-    const int col = min(n0 + (lane & 31) * 8, N - 8);
+    const int q = wave * Tile::B_DMA + j;              // 1 KB slot of the B stage: 2 k-rows x 32 chunks (4 x 16)
+    constexpr int RC = Tile::B_ROW_CHUNKS;
+    const int kr = q * (64 / RC) + lane / RC;
+    const int col = min(n0 + b_swizzle<NJ>(lane % RC, kr) * 8, N - 8);
     b_off[j] = ((uint32_t)kr * (uint32_t)N + (uint32_t)col) * 2u;
   }
   const int nk = K / kHBK;
@@ -173,15 +190,16 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
                                                16, b_off[j], ktc * kHBK * N * 2, 0, 0);
   };
 
-  float4v acc[MI][8];
+  float4v acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  // LDS read offsets in bytes: A row (wm*16*MI + i*16 + l16), chunk g (swizzled); B k-row g*8+kk, 8 columns
+  // LDS read offsets in bytes: A row (wm*16*MI + i*16 + l16), chunk g (swizzled); B k-row g*8+kk, NJ columns
   const int a_rd = ((wm * 16 * MI + l16) * 4 + (g ^ a_swizzle(l16))) * 16;
-  const int b_rd = ((g * 8) * BN + wn * 128 + l16 * 8) * 2;
+  const int b_rd = NJ == 8 ? ((g * 8) * BN + wn * 128 + l16 * 8) * 2
+                           : (g * 8) * BN * 2 + b_swizzle<NJ>(wn * 8 + (l16 >> 1), g * 8) * 16 + (l16 & 1) * 8;
 
 #pragma unroll
   for (int q = 0; q < kStages; ++q) issue(q);
@@ -189,46 +207,47 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
   barrier_only();
   // Two operand register sets: a k-step multiplies out of one while it fills the other, and the k loop below is
   // unrolled by two so that neither set is ever copied.
-  half8 a_reg[2][MI], b_reg[2][8];
+  half8 a_reg[2][MI], b_reg[2][NJ];
   {
-    uint4v raw[8];
+    Raw raw[8];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint4v*>(smem + Tile::A_BYTES + b_rd + kk * BN * 2);
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const Raw*>(smem + Tile::A_BYTES + b_rd + kk * BN * 2);
 #pragma unroll
     for (int i = 0; i < MI; ++i) a_reg[0][i] = *reinterpret_cast<const half8*>(smem + a_rd + i * 16 * 64);
     transpose8x8(raw, b_reg[0]);
   }
 
-  auto step = [&](int kt, const half8 (&a_cur)[MI], const half8 (&bop_cur)[8], half8 (&a_n)[MI], half8 (&bop_n)[8]) {
+  auto step = [&](int kt, const half8 (&a_cur)[MI], const half8 (&bop_cur)[NJ], half8 (&a_n)[MI], half8 (&bop_n)[NJ]) {
     wait_vmcnt<Tile::DMA * (kStages - 2)>();   // k-step kt+1 has landed; kt+2 and kt+3 may still be in flight
     wait_lgkmcnt0();                           // this wavefront's reads of k-step kt's buffer are complete
     barrier_only();
     issue(kt + kStages);                       // into the buffer of k-step kt, free now for every wavefront
     const unsigned char* st = smem + ((kt + 1) % kStages) * Tile::STAGE_BYTES;
-    uint4v raw[8];
+    Raw raw[8];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const uint4v*>(st + Tile::A_BYTES + b_rd + kk * BN * 2);
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *reinterpret_cast<const Raw*>(st + Tile::A_BYTES + b_rd + kk * BN * 2);
 #pragma unroll
     for (int i = 0; i < MI; ++i) a_n[i] = *reinterpret_cast<const half8*>(st + a_rd + i * 16 * 64);
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
+      for (int j = 0; j < NJ; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[i], bop_cur[j], acc[i][j], 0, 0, 0);
     transpose8x8(raw, bop_n);
     // issue order: the MFMAs start right behind the barrier; the LDS reads and this wave's DMA instructions go between
     // the first of them, the transposes (which wait for the reads) between the rest
-    constexpr int kReads = 8 + MI, kMfma = 8 * MI, kLate = kMfma - kReads;
+    constexpr int kReads = 8 + MI, kMfma = NJ * MI, kPerms = 4 * NJ;
+    constexpr int kEarly = kReads < kMfma / 2 ? kReads : kMfma / 2, kLate = kMfma - kEarly;
 #pragma unroll
-    for (int r = 0; r < kReads; ++r) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 LDS read
-      if (r < Tile::DMA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 DMA instruction
+    for (int r = 0; r < kEarly; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kEarly - 1) / kEarly, 0);        // its share of the LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x020, (Tile::DMA + kEarly - 1) / kEarly, 0);     // and of the DMA instructions
     }
 #pragma unroll
     for (int r = 0; r < kLate; ++r) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x002, (32 + kLate - 1) / kLate, 0);   // its share of the 32 transposes
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                            // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, (kPerms + kLate - 1) / kLate, 0);   // its share of the transposes
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -241,26 +260,26 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
   if (kt < nk) step(kt, a_reg[0], b_reg[0], a_reg[1], b_reg[1]);
   wait_vmcnt<0>();        // no DMA may still target this workgroup's LDS when it ends
 
-  // epilogue: lane owns rows g*4+r of every 16-row sub-tile and 8 consecutive columns
-  const int col = n0 + wn * 128 + l16 * 8;
+  // epilogue: lane owns rows g*4+r of every 16-row sub-tile and NJ consecutive columns
+  const int col = n0 + wn * (BN / 2) + l16 * NJ;
   if (col < N) {
     _Float16* C = (_Float16*)args.C + (size_t)grp * N + col;
-    half8 bias8;
+    HalfN bias8;
     const bool has_bias = args.bias[grp] != nullptr;
-    if (has_bias) bias8 = *reinterpret_cast<const half8*>((const _Float16*)args.bias[grp] + col);
+    if (has_bias) bias8 = *reinterpret_cast<const HalfN*>((const _Float16*)args.bias[grp] + col);
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = m0 + wm * 16 * MI + i * 16 + g * 4 + r;
         if (row < rows) {
-          half8 o;
+          HalfN o;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) o[j] = f2h(acc[i][j][r]);
+          for (int j = 0; j < NJ; ++j) o[j] = f2h(acc[i][j][r]);
           // half add on the rounded product, as the reference's next kernel does; optionally that kernel's GELU too
-          if (args.gelu) o = bias_gelu_half<half8, 8>(o, bias8);
+          if (args.gelu) o = bias_gelu_half<HalfN, NJ>(o, bias8);
           else if (has_bias) o = o + bias8;
-          __builtin_nontemporal_store(o, reinterpret_cast<half8*>(C + (size_t)row * args.ldc));
+          __builtin_nontemporal_store(o, reinterpret_cast<HalfN*>(C + (size_t)row * args.ldc));
         }
       }
   }
@@ -291,7 +310,6 @@ constexpr int kPStage = (kPBM * kHBK + kHBK * kPBN) * 2;      // 32 KB per k-ste
 constexpr int kPSmem = kStages * kPStage;                     // 128 KB
 [[maybe_unused]] constexpr int kPABytes = kPBM * kHBK * 2;     // A part of a k-step slot, B follows
 
-typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 struct PTile {
   int m0, n0, grp;
@@ -831,13 +849,13 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
   }
 }
 
-template <int MI>
+template <int MI, int NJ>
 void launch_f16(GemmArgs a, hipStream_t stream) {
-  using Tile = HTile<MI>;
-  auto kern = gemm_f16_kernel<MI>;
+  using Tile = HTile<MI, NJ>;
+  auto kern = gemm_f16_kernel<MI, NJ>;
   allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Tile::SMEM_BYTES);
   a.tiles_m = (a.m_bound + Tile::BM - 1) / Tile::BM;
-  a.tiles_n = (a.n + kHBN - 1) / kHBN;
+  a.tiles_n = (a.n + Tile::BN - 1) / Tile::BN;
   const int total = a.tiles_m * a.tiles_n * a.groups;
   a.per_xcd = (total + kXcds - 1) / kXcds;
   kern<<<a.per_xcd * kXcds, kHThreads, Tile::SMEM_BYTES, stream>>>(a);
@@ -985,9 +1003,11 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
     } else {
       // less than a round of tiles: the time is the latency of one tile's k loop, which is shorter for 64-row tiles
       // (two of their workgroups fit a CU); from about two tiles per CU on the 128-row tile is the better one
-      const long small = (long)((m_bound + 63) / 64) * ((n + kHBN - 1) / kHBN) * g.groups;
-      if (small <= 2L * device_cu_count()) launch_f16<2>(a, stream);
-      else launch_f16<4>(a, stream);
+      const long small = (long)((m_bound + 63) / 64) * ((n + 255) / 256) * g.groups;
+      // fewer 64 x 256 tiles than CUs: the k loop runs at the rate one CU's DMA fills its LDS, so halve the tile
+      if (small <= device_cu_count() && n % 8 == 0 && n >= 128) launch_f16<2, 4>(a, stream);
+      else if (small <= 2L * device_cu_count()) launch_f16<2, 8>(a, stream);
+      else launch_f16<4, 8>(a, stream);
     }
   } else {
     // less than a round of 128x128 tiles: 64x64 tiles finish their k loop four times sooner

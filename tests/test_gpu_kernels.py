@@ -294,7 +294,8 @@ def test_fused_attention_many_sequences_head_groups(k, dtype):
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 @pytest.mark.parametrize("m,n,k_", [(1, 768, 768), (134, 768, 768), (257, 3072, 768), (300, 768, 3072),
-                                    (1000, 1024, 1024), (100, 200, 64), (70, 264, 128), (2000, 2304, 768)])
+                                    (1000, 1024, 1024), (100, 200, 64), (70, 264, 128), (2000, 2304, 768),
+                                    (5000, 3072, 96), (40, 136, 64)])
 def test_gemm(k, dtype, m, n, k_):
     print("gemm", dtype, m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_)
@@ -345,9 +346,10 @@ def test_gemm_bt(k, m, n, k_):
     assert np.array_equal(got2[:m - 301], got[:m - 301]) and np.all(got2[m - 301:] == 0)
 
 
-# every GEMM kernel behind et_gemm: fp32 128x128 and 64x64 tiles, fp16 64- and 128-row tiles, fp16 persistent
+# every GEMM kernel behind et_gemm: fp32 128x128 and 64x64 tiles, fp16 64x128, 64x256 and 128x256 tiles, fp16 persistent
 @pytest.mark.parametrize("dtype,m,n,k_", [("fp32", 700, 256, 64), ("fp32", 3000, 3072, 96), ("fp16", 300, 512, 64),
-                                           ("fp16", 5000, 3072, 96), ("fp16", 11000, 1032, 160)])
+                                           ("fp16", 2000, 2304, 64), ("fp16", 5000, 3072, 96),
+                                           ("fp16", 11000, 1032, 160)])
 def test_gemm_bias_gelu_equals_the_two_passes(k, dtype, m, n, k_):
     print("gemm_bias_gelu", dtype, m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_ + 2)
