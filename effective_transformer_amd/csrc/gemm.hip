@@ -735,6 +735,7 @@ constexpr int kFAStride = kFBK + 4;       // floats; 80-byte rows
 // round of 128x128 tiles, where the time is the k loop of one tile: a quarter of the MFMAs per k-step)
 template <int WB>
 __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
+#if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   constexpr int kFBM = 64 * WB, kFBN = 64 * WB;
   constexpr size_t kFABytes = (size_t)kFBM * kFAStride * 4;
   constexpr size_t kFBBytes = (size_t)kFBK * kFBN * 4;
@@ -753,8 +754,12 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
   const int m0 = tm * kFBM;
   const int n0 = tn * kFBN;
   const int N = args.n, K = args.k;
-  const float* __restrict__ A = (const float*)args.A[grp];
-  const float* __restrict__ B = (const float*)args.B[grp];
+  // Loads go through buffer descriptors: rows at or beyond the valid count and columns at or beyond n read as zero
+  // without a branch, so every k-step issues the same number of loads and the waits can count them.
+  __amdgpu_buffer_rsrc_t rsrc_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(args.A[grp]), 0, (int)((uint32_t)rows * K * 4u), 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_b =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(args.B[grp]), 0, (int)((uint32_t)K * N * 4u), 0x00020000);
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -762,22 +767,32 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, kb = lane >> 5;
 
-  u32x4 ra[WB], rb[WB];
+  // Global -> registers -> LDS.  The 64 x 64 tile runs where few workgroups are resident and nothing else hides the
+  // latency of a global load, so its k-steps are requested kDepth steps ahead (a ring of register sets); the big tile
+  // has three wavefronts per SIMD for that and keeps one set.
+  constexpr int kDepth = WB == 1 ? 4 : 1;
+  u32x4 ring_a[kDepth][WB], ring_b[kDepth][WB];
   const int a_kc = tid & 3, a_row = tid >> 2;                // + u*64
   const int b_nc = tid % kBc4, b_krow = tid / kBc4;          // + u*kBRows
   const bool b_col_ok = n0 + b_nc * 4 < N;
+  uint32_t a_off[WB], b_off[WB];      // byte offsets of this thread's pieces at k = 0; the range check looks at these
+#pragma unroll
+  for (int u = 0; u < WB; ++u) {
+    a_off[u] = ((uint32_t)(m0 + a_row + u * 64) * (uint32_t)K + (uint32_t)a_kc * 4u) * 4u;
+    b_off[u] = ((uint32_t)(b_krow + u * kBRows) * (uint32_t)N + (uint32_t)(n0 + b_nc * 4)) * 4u;
+  }
+  const int nk = K / kFBK;
 
-  auto load_global = [&](int k0) {
+  auto load_global = [&](int kt, u32x4 (&ra)[WB], u32x4 (&rb)[WB]) {
+    const int k0 = min(kt, nk - 1) * kFBK;    // past the end: the last k-step again (never used; keeps the load count uniform)
 #pragma unroll
     for (int u = 0; u < WB; ++u) {
-      const int row = m0 + a_row + u * 64;
-      ra[u] = u32x4{0u, 0u, 0u, 0u};
-      if (row < rows) ra[u] = *reinterpret_cast<const u32x4*>(A + (size_t)row * K + k0 + a_kc * 4);
-      rb[u] = u32x4{0u, 0u, 0u, 0u};
-      if (b_col_ok) rb[u] = *reinterpret_cast<const u32x4*>(B + (size_t)(k0 + b_krow + u * kBRows) * N + n0 + b_nc * 4);
+      ra[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, a_off[u], k0 * 4, 0));
+      const uint32_t off = b_col_ok ? b_off[u] + (uint32_t)k0 * (uint32_t)N * 4u : 0xffffffffu;
+      rb[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, off, 0, 0));
     }
   };
-  auto store_lds = [&](int stage) {
+  auto store_lds = [&](int stage, const u32x4 (&ra)[WB], const u32x4 (&rb)[WB]) {
     float* As = reinterpret_cast<float*>(smem + stage * kFStage);
     float* Bs = reinterpret_cast<float*>(smem + stage * kFStage + kFABytes);
 #pragma unroll
@@ -795,39 +810,46 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int nk = K / kFBK;
-  load_global(0);
-  store_lds(0);
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) load_global(d, ring_a[d], ring_b[d]);
+  store_lds(0, ring_a[0], ring_b[0]);
+  load_global(kDepth, ring_a[0], ring_b[0]);
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    if (kt + 1 < nk) load_global((kt + 1) * kFBK);
-    const float* As = reinterpret_cast<const float*>(smem + (kt & 1) * kFStage);
-    const float* Bs = reinterpret_cast<const float*>(smem + (kt & 1) * kFStage + kFABytes);
-    // step s of the stage contracts k = kb*8 + s (the same choice for A and B)
-    float a[WB][8], b[WB][8];
+  for (int kt0 = 0; kt0 < nk; kt0 += kDepth) {
 #pragma unroll
-    for (int i = 0; i < WB; ++i) {
-      const float* ap = As + (wm * 32 * WB + i * 32 + l32) * kFAStride + kb * 8;
-      const float4v a0 = *reinterpret_cast<const float4v*>(ap);
-      const float4v a1 = *reinterpret_cast<const float4v*>(ap + 4);
+    for (int d = 0; d < kDepth; ++d) {
+      const int kt = kt0 + d;
+      if (kt >= nk) break;
+      const float* As = reinterpret_cast<const float*>(smem + (kt & 1) * kFStage);
+      const float* Bs = reinterpret_cast<const float*>(smem + (kt & 1) * kFStage + kFABytes);
+      // step s of the stage contracts k = kb*8 + s (the same choice for A and B)
+      float a[WB][8], b[WB][8];
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        a[i][s] = a0[s];
-        a[i][4 + s] = a1[s];
+      for (int i = 0; i < WB; ++i) {
+        const float* ap = As + (wm * 32 * WB + i * 32 + l32) * kFAStride + kb * 8;
+        const float4v a0 = *reinterpret_cast<const float4v*>(ap);
+        const float4v a1 = *reinterpret_cast<const float4v*>(ap + 4);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          a[i][s] = a0[s];
+          a[i][4 + s] = a1[s];
+        }
       }
+#pragma unroll
+      for (int j = 0; j < WB; ++j)
+#pragma unroll
+        for (int s = 0; s < 8; ++s) b[j][s] = Bs[(kb * 8 + s) * kFBN + wn * 32 * WB + j * 32 + l32];
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+#pragma unroll
+        for (int i = 0; i < WB; ++i)
+#pragma unroll
+          for (int j = 0; j < WB; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+      // k-step kt+1 sits in ring slot (kt+1) % kDepth = (d+1) % kDepth; once it is in LDS the slot takes k-step kt+1+kDepth
+      store_lds((kt + 1) & 1, ring_a[(d + 1) % kDepth], ring_b[(d + 1) % kDepth]);
+      load_global(kt + 1 + kDepth, ring_a[(d + 1) % kDepth], ring_b[(d + 1) % kDepth]);
+      __syncthreads();
     }
-#pragma unroll
-    for (int j = 0; j < WB; ++j)
-#pragma unroll
-      for (int s = 0; s < 8; ++s) b[j][s] = Bs[(kb * 8 + s) * kFBN + wn * 32 * WB + j * 32 + l32];
-#pragma unroll
-    for (int s = 0; s < 8; ++s)
-#pragma unroll
-      for (int i = 0; i < WB; ++i)
-#pragma unroll
-        for (int j = 0; j < WB; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
-    if (kt + 1 < nk) store_lds((kt + 1) & 1);
-    __syncthreads();
   }
 
 #pragma unroll
@@ -847,6 +869,9 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
         }
       }
   }
+#else
+  (void)args;
+#endif
 }
 
 template <int MI, int NJ>
