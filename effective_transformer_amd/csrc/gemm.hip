@@ -770,7 +770,7 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
   // Global -> registers -> LDS.  The 64 x 64 tile runs where few workgroups are resident and nothing else hides the
   // latency of a global load, so its k-steps are requested kDepth steps ahead (a ring of register sets); the big tile
   // has three wavefronts per SIMD for that and keeps one set.
-  constexpr int kDepth = WB == 1 ? 4 : 1;
+  constexpr int kDepth = WB == 1 ? 4 : 2;
   u32x4 ring_a[kDepth][WB], ring_b[kDepth][WB];
   const int a_kc = tid & 3, a_row = tid >> 2;                // + u*64
   const int b_nc = tid % kBc4, b_krow = tid / kBc4;          // + u*kBRows
