@@ -1026,12 +1026,12 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
     if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
       launch_f16_persistent(a, stream, g.b_transposed);
     } else {
-      // less than a round of tiles: the time is the latency of one tile's k loop, which is shorter for 64-row tiles
-      // (two of their workgroups fit a CU); from about two tiles per CU on the 128-row tile is the better one
+      // Below a round of the chip the time of a launch is the k loop of one tile.  With fewer 64 x 256 tiles than CUs
+      // that loop runs at the rate one CU's DMA fills its LDS: the 64 x 128 tile halves the B bytes per workgroup and
+      // doubles the workgroups.  From there on the 128 x 256 tile is the faster one (measured at n = 768 .. 3072,
+      // k = 768 and 3072; a 64 x 256 tile never won between the two).
       const long small = (long)((m_bound + 63) / 64) * ((n + 255) / 256) * g.groups;
-      // fewer 64 x 256 tiles than CUs: the k loop runs at the rate one CU's DMA fills its LDS, so halve the tile
-      if (small <= device_cu_count() && n % 8 == 0 && n >= 128) launch_f16<2, 4>(a, stream);
-      else if (small <= 2L * device_cu_count()) launch_f16<2, 8>(a, stream);
+      if (small <= device_cu_count()) launch_f16<2, 4>(a, stream);
       else launch_f16<4, 8>(a, stream);
     }
   } else {

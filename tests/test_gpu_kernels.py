@@ -346,7 +346,7 @@ def test_gemm_bt(k, m, n, k_):
     assert np.array_equal(got2[:m - 301], got[:m - 301]) and np.all(got2[m - 301:] == 0)
 
 
-# every GEMM kernel behind et_gemm: fp32 128x128 and 64x64 tiles, fp16 64x128, 64x256 and 128x256 tiles, fp16 persistent
+# every GEMM kernel behind et_gemm: fp32 128x128 and 64x64 tiles, fp16 64x128 and 128x256 tiles, fp16 persistent
 @pytest.mark.parametrize("dtype,m,n,k_", [("fp32", 700, 256, 64), ("fp32", 3000, 3072, 96), ("fp16", 300, 512, 64),
                                            ("fp16", 2000, 2304, 64), ("fp16", 5000, 3072, 96),
                                            ("fp16", 11000, 1032, 160)])
