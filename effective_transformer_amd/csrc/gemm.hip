@@ -15,6 +15,7 @@
 // The M dimension (valid tokens) may live on the device: tiles beyond *rows_dev exit, the last tile
 // is predicated.  Up to three column groups (Q/K/V) share one launch.
 #include <algorithm>
+#include <atomic>
 
 #include <type_traits>
 
@@ -729,7 +730,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
 // ------------------------------------------------------------------------------------------
 constexpr int kFThreads = 256;
 constexpr int kFBK = 16;
-constexpr int kFAStride = kFBK + 4;       // floats; 80-byte rows
+[[maybe_unused]] constexpr int kFAStride = kFBK + 4;       // floats; 80-byte rows
 
 // WB = 32x32 MFMA blocks per wavefront and dimension: 2 -> 128x128 tile, 1 -> 64x64 tile (problems of less than a
 // round of 128x128 tiles, where the time is the k loop of one tile: a quarter of the MFMAs per k-step)
@@ -888,14 +889,16 @@ void launch_f16(GemmArgs a, hipStream_t stream) {
 
 int device_cu_count() {
   constexpr int kMaxDevices = 64;
-  static int cus[kMaxDevices] = {};
+  static std::atomic<int> cus[kMaxDevices] = {};      // handles on several GPUs may launch from different threads
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-  if (cus[dev] == 0) {
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     hipDeviceProp_t prop;
-    cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    n = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  return cus[dev];
+  return n;
 }
 
 void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
