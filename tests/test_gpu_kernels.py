@@ -346,6 +346,27 @@ def test_gemm_bt(k, m, n, k_):
     assert np.array_equal(got2[:m - 301], got[:m - 301]) and np.all(got2[m - 301:] == 0)
 
 
+# A sequence gives the same bits in a batch of any size: every fp16 kernel accumulates k in the same order, so the
+# rows of a small problem (64x128 tiles), a middle one (128x256 tiles) and a large one (persistent 256x256 tiles, B in
+# either storage order) agree bit for bit; the two fp32 tiles likewise.
+@pytest.mark.parametrize("n,k_", [(768, 768), (768, 3072), (3072, 768)])
+def test_gemm_same_bits_in_every_kernel(k, n, k_):
+    print("gemm same bits", n, k_, flush=True)
+    rng = np.random.RandomState(n + k_)
+    m = 11000
+    a = dev(o.rnd(rng.randn(m, k_), "fp16"))
+    b = dev(o.rnd(0.05 * rng.randn(k_, n), "fp16"))
+    big = k.gemm(a, b).cpu().numpy()
+    assert np.array_equal(k.gemm_bt(a, k.transpose_weight(b)).cpu().numpy(), big)
+    for rows in (6000, 2500, 300, 1):
+        part = k.gemm(a[:rows].contiguous(), b).cpu().numpy()
+        assert np.array_equal(part, big[:rows]), rows
+    a32, b32 = a.float(), b.float()
+    big32 = k.gemm(a32, b32).cpu().numpy()
+    for rows in (1500, 100):
+        assert np.array_equal(k.gemm(a32[:rows].contiguous(), b32).cpu().numpy(), big32[:rows]), rows
+
+
 # every GEMM kernel behind et_gemm: fp32 128x128 and 64x64 tiles, fp16 64x128 and 128x256 tiles, fp16 persistent
 @pytest.mark.parametrize("dtype,m,n,k_", [("fp32", 700, 256, 64), ("fp32", 3000, 3072, 96), ("fp16", 300, 512, 64),
                                            ("fp16", 2000, 2304, 64), ("fp16", 5000, 3072, 96),
