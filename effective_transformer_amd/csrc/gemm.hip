@@ -776,6 +776,9 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
   const int a_kc = tid & 3, a_row = tid >> 2;                // + u*64
   const int b_nc = tid % kBc4, b_krow = tid / kBc4;          // + u*kBRows
   const bool b_col_ok = n0 + b_nc * 4 < N;
+  // offset of a lane whose columns do not exist: beyond any B this kernel accepts (k*n*4 < 2 GB) and far enough from
+  // 2^32 that offset + access size cannot wrap, so the range check zero-fills it
+  constexpr uint32_t kBeyondB = 0x80000000u;
   uint32_t a_off[WB], b_off[WB];      // byte offsets of this thread's pieces at k = 0; the range check looks at these
 #pragma unroll
   for (int u = 0; u < WB; ++u) {
@@ -789,7 +792,7 @@ __global__ __launch_bounds__(kFThreads, 4) void gemm_f32_kernel(GemmArgs args) {
 #pragma unroll
     for (int u = 0; u < WB; ++u) {
       ra[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, a_off[u], k0 * 4, 0));
-      const uint32_t off = b_col_ok ? b_off[u] + (uint32_t)k0 * (uint32_t)N * 4u : 0xffffffffu;
+      const uint32_t off = b_col_ok ? b_off[u] + (uint32_t)k0 * (uint32_t)N * 4u : kBeyondB;
       rb[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, off, 0, 0));
     }
   };
@@ -1005,7 +1008,7 @@ void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, con
 bool gemm_supported(DType t, int n, int k, int groups) {
   if (groups < 1 || groups > 3 || n <= 0 || k <= 0) return false;
   if (t == DType::F16) return k % kHBK == 0 && n % 8 == 0 && n >= 8;
-  return k % kFBK == 0 && n % 4 == 0;
+  return k % kFBK == 0 && n % 4 == 0 && (uint64_t)k * (uint64_t)n * 4u < 0x80000000ull;
 }
 
 void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k, const int32_t* rows_dev,
