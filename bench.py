@@ -4,7 +4,8 @@
 
 A step is one pass Input -> L x Layer -> Output over one synthetic batch that is already
 resident in HBM.  Prints ONE JSON line: valid tokens/s (whole job), ms/step, the roofline of the
-dominant kernel measured live with HIP events, per-kernel rooflines, and the CPU baseline (the
+dominant kernel measured live with HIP events (inside the layer's launch sequence, and in a launch loop of the
+kernel alone), per-kernel rooflines, and the CPU baseline (the
 standard padded BERT encoder graph on the host cores, on a bounded sample of the same batch).
 """
 import argparse
@@ -157,6 +158,82 @@ def per_kernel(wl, T, mask_np, iters=20):
     return res
 
 
+def in_layer_kernels(wl, T, mask_np, reps=4):
+    """The kernels of one layer launched in the layer's own order on the layer's own data flow (each kernel reads what
+    the one before it wrote, as inside et_layer), with a HIP event between every two launches: the duration a kernel
+    has on the path, where its input is still in the last-level cache.  Returns ms per launch by kernel name and the
+    sum over one layer."""
+    import torch
+    from effective_transformer_amd import kernel_ops as k, ops
+
+    dt = torch.float16 if wl.dtype == "fp16" else torch.float32
+    B, S, H, F, heads, d = wl.B, wl.S, wl.H, wl.F, wl.heads, wl.d
+    g = torch.Generator(device="cuda").manual_seed(1)
+    rnd = lambda *s: torch.randn(*s, device="cuda", dtype=torch.float32, generator=g).to(dt)
+    mask = torch.from_numpy(mask_np).cuda()
+    attr = mask[:, None, :].expand(B, S, S).to(dt).contiguous()
+    x, vwn, bidx, widx = ops.effective_transformer_input(rnd(B, S, H), mask, B, S, S, heads, d)
+    x = x.reshape(B * S, H)[:T]
+    weights = {"gemm_qkv": rnd(H, 3 * H) * 0.02, "gemm_attn_out": rnd(H, H) * 0.02, "gemm_ffn_up": rnd(H, F) * 0.02,
+               "gemm_ffn_down": rnd(F, H) * 0.02}
+    bias = {n: rnd(w.shape[1]) * 0.02 for n, w in weights.items()}
+    gam, bet = torch.ones(H, device="cuda", dtype=dt), torch.zeros(H, device="cuda", dtype=dt)
+    mm = {}
+    for n, w in weights.items():          # the kernel the encoder object runs this projection on
+        mm[n] = (k.gemm, w)
+        if dt == torch.float16:
+            wt = k.transpose_weight(w)
+            try:
+                k.gemm_bt(rnd(T, w.shape[0]), wt)
+                mm[n] = (k.gemm_bt, wt)
+            except Exception:
+                pass
+    qkv = torch.empty(T, 3 * H, device="cuda", dtype=dt)
+    ctx, ao, spare = (torch.empty(T, H, device="cuda", dtype=dt) for _ in range(3))
+    inter = torch.empty(T, F, device="cuda", dtype=dt)
+    names = ("gemm_qkv", "attention", "gemm_attn_out", "bias_residual_layernorm", "gemm_ffn_up", "gemm_ffn_down",
+             "bias_residual_layernorm")
+
+    def layer(ev):
+        cur, down = x, spare
+        for l in range(wl.layers):
+            e = ev[l] if ev else None
+            f, w = mm["gemm_qkv"]
+            if e: e[0].record()
+            f(cur, w, bias=bias["gemm_qkv"], out=qkv)
+            if e: e[1].record()
+            k.attention(qkv, qkv[:, H:], qkv[:, 2 * H:], 1, 3 * H, attr, vwn, B, S, heads, d, bidx, widx, dst=ctx)
+            if e: e[2].record()
+            f, w = mm["gemm_attn_out"]
+            f(ctx, w, out=ao)
+            if e: e[3].record()
+            k.add_bias_input_layernorm(ao, cur, bias["gemm_attn_out"], gam, bet)
+            if e: e[4].record()
+            f, w = mm["gemm_ffn_up"]
+            f(ao, w, bias=bias["gemm_ffn_up"], gelu=True, out=inter)
+            if e: e[5].record()
+            f, w = mm["gemm_ffn_down"]
+            f(inter, w, out=down)
+            if e: e[6].record()
+            k.add_bias_input_layernorm(down, ao, bias["gemm_ffn_down"], gam, bet)
+            if e: e[7].record()
+            cur, down = down, cur      # the layer's output feeds the next layer
+
+    layer(None)
+    tot = {n: 0.0 for n in names}
+    for _ in range(reps):
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(8)] for _ in range(wl.layers)]
+        torch.cuda.synchronize()
+        layer(ev)
+        torch.cuda.synchronize()
+        for e in ev:
+            for i, n in enumerate(names):
+                tot[n] += e[i].elapsed_time(e[i + 1])
+    calls = {n: reps * wl.layers * names.count(n) for n in tot}
+    per = {n: tot[n] / calls[n] for n in tot}
+    return per, sum(per[n] * names.count(n) for n in per)
+
+
 def cpu_baseline(w, nseq=0, budget_s=12.0):
     """The standard padded BERT encoder graph (the reference's comparison path) in fp32 on the host cores, all
     layers, on the first `nseq` sequences of the batch.  nseq = 0: as many sequences as fit about `budget_s`
@@ -255,15 +332,35 @@ def main():
         del g
     kernels = {} if a.no_kernels else per_kernel(wl, T, w["mask"])
     roof = None
+    layer_sum = None
     if kernels:
-        # dominant kernel = the largest share of a layer's time
-        share = {n: v["ms"] for n, v in kernels.items() if n.startswith("gemm") or n == "attention"}
-        share["bias_residual_layernorm"] = 2 * kernels["bias_residual_layernorm"]["ms"]
+        # the same kernels inside the layer's launch sequence: what each costs on the path
+        per, layer_sum = in_layer_kernels(wl, T, w["mask"])
+        # launches shorter than the host's time per call space the events by the host, not by the GPU: then the sum
+        # over the layers exceeds the measured step and the launch loop of the kernel alone is the better clock
+        host_bound = layer_sum * wl.layers > 1.05 * ms
+        for n, ms_l in per.items():
+            kd = kernels[n]
+            kd["ms_in_layer"] = round(ms_l, 5)
+            kd["achieved_in_layer"] = round(kd["achieved"] * kd["ms"] / ms_l, 2)
+            kd["frac_in_layer"] = round(kd["achieved_in_layer"] / kd["peak"], 4)
+        # dominant kernel = the largest share of a layer's time; its roofline is priced at its duration on the path
+        # (the `ms` a launch loop of the kernel alone gives, with cold inputs, stays beside it)
+        share = {n: (kernels[n]["ms"] if host_bound else per[n]) * (2 if n == "bias_residual_layernorm" else 1)
+                 for n in per}
         dom = max(share, key=share.get)
         kd = kernels[dom]
-        roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved"], "peak": kd["peak"], "unit": kd["unit"],
-                "frac": kd["frac"], "ms": kd["ms"],
-                "traffic": MEASURED_TRAFFIC.get((wl.name, dom))}
+        alone = {"ms": kd["ms"], "achieved": kd["achieved"], "frac": kd["frac"]}
+        if host_bound:
+            roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved"], "peak": kd["peak"],
+                    "unit": kd["unit"], "frac": kd["frac"], "ms": kd["ms"],
+                    "measured": "HIP events around a launch loop of the kernel alone (the layer replica is host-bound at this size)",
+                    "traffic": MEASURED_TRAFFIC.get((wl.name, dom))}
+        else:
+            roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved_in_layer"], "peak": kd["peak"],
+                    "unit": kd["unit"], "frac": kd["frac_in_layer"], "ms": kd["ms_in_layer"],
+                    "measured": "HIP events around the kernel inside the layer's launch sequence, %d launches" % (4 * wl.layers),
+                    "alone": alone, "traffic": MEASURED_TRAFFIC.get((wl.name, dom))}
     cpu = None
     if not a.no_cpu:
         cpu = cpu_baseline(w, a.cpu_seqs)
@@ -280,7 +377,8 @@ def main():
         "config": {"workload": "%s: BERT %d layers, hidden %d, %d heads x %d, FFN %d, batch %d, max_seq %d, %d valid tokens"
                                % (wl.name, wl.layers, wl.H, wl.heads, wl.d, wl.F, wl.B, wl.S, T),
                    "valid_tokens": T, "padded_tokens": wl.B * wl.S},
-        "roofline": roof, "kernels": kernels, "cpu_baseline": cpu,
+        "roofline": roof, "layer_ms_sum_of_kernels": None if layer_sum is None else round(layer_sum, 4),
+        "kernels": kernels, "cpu_baseline": cpu,
     }))
 
 
