@@ -512,9 +512,16 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
   constexpr bool PF = CPT <= 4;                // more than 4 chunks x 3 matrices in flight would not fit the registers
   auto kern = attention_kernel<T, NKT, CPT, PF>;
   allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Sm::kBytes);
-  // a workgroup serves up to 4 heads of one sequence: mask rows, positions and zero fill are shared by them
-  int hpw = 4;
-  while (hpw > 1 && (long)batch * ((heads + hpw - 1) / hpw) < 2048) hpw >>= 1;   // small batches: more workgroups
+  // A workgroup serves several heads of one sequence: mask rows, positions and zero fill are shared by them, and the
+  // chain of dependent loads a workgroup starts with (sequence start, positions, rows) is paid once.  Up to 4 heads
+  // (8 for the 128-key kernel, whose start is the longest), in equal groups, as long as about two workgroups per CU
+  // remain: measured best on batches of 100 x 32, 1000 x 64 and 256 x 128 tokens.
+  int hpw = 1;
+  for (int h = NKT >= 8 ? 8 : 4; h > 1; --h)
+    if (heads % h == 0 && (long)batch * (heads / h) >= 512) {
+      hpw = h;
+      break;
+    }
   dim3 grid((heads + hpw - 1) / hpw, batch);
   kern<<<grid, kAttnThreads, Sm::kBytes, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
                                                    (const T*)attr_mask, (T*)dst, seq_start, word_idx, seq_len, heads,
