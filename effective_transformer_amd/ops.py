@@ -16,7 +16,7 @@ import torch
 from . import _lib
 
 _handles: Dict[int, C.c_void_p] = {}
-_workspaces: Dict[Tuple[int, int, str], torch.Tensor] = {}
+_workspaces: Dict[tuple, torch.Tensor] = {}
 _lock = threading.Lock()
 
 
@@ -40,16 +40,22 @@ def handle(device: torch.device) -> C.c_void_p:
         return h
 
 
+_scope = threading.local()      # .owner: set while a GraphedEncoder warms up and captures (its buffers are its own)
+
+
 def _workspace(device: torch.device, kind: str, nbytes: int) -> torch.Tensor:
-    """One scratch buffer per (GPU, stream, kind), grown on demand: calls queued on one stream run in order and may
-    share it, calls on different streams get their own."""
+    """One scratch buffer per (GPU, stream, kind, owner), grown on demand: calls queued on one stream run in order and
+    may share it, calls on different streams get their own, and so does every captured graph (a graph keeps the
+    addresses it was captured with, and replays of two graphs on different streams may overlap).  Within one such key
+    the contract is one stream of calls: the layer op keeps its intermediate tensors there between its launches."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    key = (idx, torch.cuda.current_stream(idx).cuda_stream, kind)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    key = (idx, torch.cuda.current_stream(idx).cuda_stream, kind, getattr(_scope, "owner", None))
+    with _lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+            _workspaces[key] = ws
+        return ws
 
 
 def _stream() -> C.c_void_p:
@@ -263,7 +269,11 @@ def effective_transformer(from_tensor: torch.Tensor, to_tensor: torch.Tensor, at
                           _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B, from_seq_len, to_seq_len,
                           head_num, size_per_head, valid_word_num_hint, _p(ws), ws.numel(), _stream())
     else:
-        prep = weights.prepared if weights.prepared is not None else _lib.LayerPrepared()
+        # a copy per call: the weights object (and its prepared struct) may be shared by threads and streams, the
+        # sequence start table belongs to this batch
+        prep = _lib.LayerPrepared()
+        if weights.prepared is not None:
+            C.pointer(prep)[0] = weights.prepared
         prep.seq_start = seq_start.data_ptr() if seq_start is not None else None
         st = lib.et_layer_with_prepared(h, code, C.byref(weights.struct), C.byref(prep), _p(from_tensor), _p(to_tensor),
                                         _p(attr_mask), _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B,
@@ -403,17 +413,30 @@ class GraphedEncoder:
         self.x = from_tensor.clone()
         self.mask = input_mask.clone()
         self.attn = attention_mask.clone()
-        # warm-up outside the capture: workspaces, kernel attributes and the output buffers get created here
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(2):
-                enc(self.x, self.mask, self.attn, sync_count=False)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.out = enc(self.x, self.mask, self.attn, sync_count=False)
+        # warm-up outside the capture: workspaces, kernel attributes and the output buffers get created here.  The
+        # workspaces and the encoder's ping-pong buffers made under this owner belong to this graph alone.
+        _scope.owner = id(self)
+        saved_bufs, enc._bufs = enc._bufs, {}
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(2):
+                    enc(self.x, self.mask, self.attn, sync_count=False)
+                self._held = [ws for key, ws in list(_workspaces.items()) if key[3] == id(self)]
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.out = enc(self.x, self.mask, self.attn, sync_count=False)
+            self._held += [ws for key, ws in list(_workspaces.items()) if key[3] == id(self)]
+            self._held += [t for bufs in enc._bufs.values() for t in bufs]
+        finally:
+            _scope.owner = None
+            enc._bufs = saved_bufs
+            with _lock:
+                for key in [k for k in _workspaces if k[3] == id(self)]:
+                    del _workspaces[key]
 
     def __call__(self, from_tensor=None, input_mask=None, attention_mask=None) -> torch.Tensor:
         """Copies the given tensors into the graph's inputs (None = keep the previous ones), replays, and returns the

@@ -100,8 +100,8 @@ def main(args):
         print("max diff : {:.6}, avg diff : {:.6}.".format(float(diff.max()), float(diff.mean())))
 
         def time_inference(fn):
-            iter_num = 128
-            for _ in range(10):
+            iter_num = getattr(args, "iters", 128)            # benchmark.py:114-124: 10 warm-ups, 128 timed runs
+            for _ in range(getattr(args, "warmup", 10)):
                 fn()
             torch.cuda.synchronize()
             beg = datetime.now()
@@ -114,7 +114,9 @@ def main(args):
         print("et  cost : {:.6} ms".format(time_inference(et)))
 
 
-if __name__ == "__main__":
+def build_parser() -> argparse.ArgumentParser:
+    """The reference's flags with its defaults (sample/tensorflow/benchmark.py:129-141); --seed, --iters and --warmup
+    are additions (the reference hard-codes 128 timed runs after 10 warm-ups and draws from an unseeded generator)."""
     here = os.path.dirname(os.path.abspath(__file__))
     parser = argparse.ArgumentParser(description="Bert performance measuring sample.")
     parser.add_argument("-c", "--config", type=str, default=os.path.join(here, "bert_config.json"), help="Bert config file.")
@@ -123,4 +125,10 @@ if __name__ == "__main__":
     parser.add_argument("-m", "--max_seq_length", type=int, default=32, help="Max sequence length.")
     parser.add_argument("-a", "--avg_seq_length", type=int, default=20, help="Average sequence length.")
     parser.add_argument("--seed", type=int, default=0)
-    main(parser.parse_args())
+    parser.add_argument("--iters", type=int, default=128, help="Timed runs per model.")
+    parser.add_argument("--warmup", type=int, default=10, help="Untimed runs in front of them.")
+    return parser
+
+
+if __name__ == "__main__":
+    main(build_parser().parse_args())

@@ -46,6 +46,10 @@ def main(args):
           % (" | padded torch ms" if args.std else ""))
     print("|---|---|---|---|---|---|---|%s---|---|" % ("---|" if args.std else ""))
     for precision, max_seq, avg_seq, rows in TABLES:
+        if args.precision and precision != args.precision:
+            continue
+        if args.max_batch:
+            rows = [r for r in rows if r[0] <= args.max_batch]
         dtype = torch.float16 if precision == "fp16" else torch.float32
         rng = np.random.RandomState(args.seed)
         weights = make_weights(cfg, dtype, dev, rng)
@@ -68,11 +72,17 @@ def main(args):
         del enc, weights
 
 
-if __name__ == "__main__":
+def build_parser() -> argparse.ArgumentParser:
     here = os.path.dirname(os.path.abspath(__file__))
     parser = argparse.ArgumentParser(description="Sweep over the reference's published benchmark tables.")
     parser.add_argument("-c", "--config", type=str, default=os.path.join(here, "bert_config.json"))
     parser.add_argument("--iters", type=int, default=128)
     parser.add_argument("--std", action="store_true", help="also time the padded torch encoder")
     parser.add_argument("--seed", type=int, default=0)
-    main(parser.parse_args())
+    parser.add_argument("--precision", choices=["fp16", "fp32"], default=None, help="only the tables of this precision")
+    parser.add_argument("--max-batch", type=int, default=0, help="only rows up to this batch size (0 = all)")
+    return parser
+
+
+if __name__ == "__main__":
+    main(build_parser().parse_args())

@@ -23,9 +23,12 @@ def _check(got, want, mask, dtype):
     assert np.all(got[~valid] == 0)                              # the Output op zero-fills padding
     g, w_ = got[valid].astype(np.float64), want[valid].astype(np.float64)
     if dtype == "fp32":
-        # fp32 bar: 1e-4 relative (LayerNorm outputs are O(1); relative to max(|want|, 1))
-        err = np.abs(g - w_) / np.maximum(np.abs(w_), 1.0)
-        assert err.max() < 1e-4, err.max()
+        # fp32 bar: 1e-4 relative error of every token's output row, ||got - want|| / ||want|| (a LayerNorm output row
+        # has norm ~ sqrt(H), so no floor is needed), and 5e-5 absolute on every element.  Measured after 12 layers:
+        # 4e-6 relative per row, 1.2e-5 absolute; a drift towards the bars shows up here long before the contract breaks.
+        rel = np.linalg.norm(g - w_, axis=-1) / np.linalg.norm(w_, axis=-1)
+        assert rel.max() < 1e-4, rel.max()
+        assert np.abs(g - w_).max() < 5e-5, np.abs(g - w_).max()
     else:
         # fp16 bar: 2e-2 max-abs after 12 layers
         assert np.abs(g - w_).max() < 2e-2, np.abs(g - w_).max()
@@ -117,6 +120,75 @@ def test_prepared_q_k_v_go_together():
     enc.layers[0].prepared.attr_kernel_K_t = None
     with pytest.raises(_lib.EtError, match="go together"):
         enc(dev(w["x"], torch.float16), dev(w["mask"].astype(np.int32)), dev(w["attr_mask"], torch.float16))
+
+
+def _packed(w, x_np, dt):
+    """Input op on x_np with the workload's mask: packed tensor + the index tensors."""
+    from effective_transformer_amd import ops
+    wl = w["wl"]
+    return ops.effective_transformer_input(dev(x_np, dt), dev(w["mask"].astype(np.int32)), wl.B, wl.S, wl.S, wl.heads,
+                                           wl.d, return_host_count=True)
+
+
+@pytest.mark.parametrize("name,nseq", [("cfg1", None), ("cfg2", None), ("cfg3", 110), ("cfg4", 40)])
+@pytest.mark.parametrize("prepared", [False, True])
+@pytest.mark.parametrize("hint", [True, False])
+def test_layer_with_distinct_from_and_to_tensors(name, nseq, prepared, hint):
+    """Q comes from from_tensor, K and V from to_tensor, and the residual of the first LayerNorm is from_tensor
+    (tf_op/bert_transformer_op.cu.cc:110-141, 210): one layer with two different packed tensors against the oracle,
+    through et_layer and et_layer_with_prepared, with and without the host-side token count.  cfg3's subset is large
+    enough for the persistent large-M GEMMs (grouped Q/K/V launch with two different A operands)."""
+    from effective_transformer_amd import ops
+    print("from != to", name, "prepared", prepared, "hint", hint, flush=True)
+    w = o.make_workload(name, layers=1, random_affine=True)
+    if nseq is not None:
+        w = subset_workload(w, np.arange(nseq))
+    wl = w["wl"]
+    dt = TDT[wl.dtype]
+    rng = np.random.RandomState(99)
+    x_to = o.rnd(rng.randn(*w["x"].shape), wl.dtype)
+    frm, vwn, bidx, widx, T = _packed(w, w["x"], dt)
+    to = _packed(w, x_to, dt)[0]
+    lw = ops.LayerWeights.from_slots(frm.device, dt, w["weights"][:16])
+    if prepared:
+        lw.prepare()
+    starts = ops.sequence_starts(vwn, bidx, wl.B, wl.S) if prepared else None
+    attr = dev(w["attr_mask"], dt)
+    run = lambda a, b: ops.effective_transformer(a, b, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S, wl.heads, wl.d,
+                                                 valid_word_num_hint=T if hint else -1, seq_start=starts)
+    got = run(frm, to).reshape(wl.B * wl.S, wl.H)[:T].cpu().numpy().astype(np.float64)
+    bi, wi_ = bidx.cpu().numpy().ravel(), widx.cpu().numpy().ravel()
+    pf = frm.reshape(wl.B * wl.S, wl.H).cpu().numpy()
+    pt = to.reshape(wl.B * wl.S, wl.H).cpu().numpy()
+    want = o.layer(pf, pt, w["attr_mask"], T, bi, wi_, w["weights"][:16], wl.B, wl.S, wl.heads, wl.d,
+                   wl.dtype).astype(np.float64)
+    err = np.abs(got - want).max()
+    print("  max abs diff", err, flush=True)
+    # one layer: fp32 2e-5 absolute (measured 3e-6), fp16 4 half-ulps of an O(1) LayerNorm output (measured 2e-3)
+    assert err < (2e-5 if wl.dtype == "fp32" else 4e-3), err
+    # the check can tell the operands apart: swapped, or the same tensor twice, is far from the oracle
+    for a, b in ((to, frm), (frm, frm), (to, to)):
+        other = run(a, b).reshape(wl.B * wl.S, wl.H)[:T].cpu().numpy().astype(np.float64)
+        assert np.abs(other - want).max() > 0.1
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_get_sequence_output_is_the_encoder(dtype):
+    """The one name the reference's Python package exports (python/effective_transformer/__init__.py:32-84), with its
+    argument list and a BertConfig-like object: same result as the encoder object, and oracle parity."""
+    from types import SimpleNamespace
+    from effective_transformer_amd import get_sequence_output
+    print("get_sequence_output", dtype, flush=True)
+    w = o.make_workload("cfg1" if dtype == "fp32" else "cfg2", layers=2, random_affine=True)
+    wl = w["wl"]
+    dt = TDT[dtype]
+    config = SimpleNamespace(num_attention_heads=wl.heads, hidden_size=wl.H, num_hidden_layers=2)
+    x = dev(w["x"], dt); mask = dev(w["mask"].astype(np.int32)); attr = dev(w["attr_mask"], dt)
+    got = get_sequence_output(config=config, max_batch_size=wl.B, max_seq_length=wl.S, attention_mask=attr,
+                              input_mask=mask, from_tensor=x, weights_value=w["weights"][:32])
+    assert tuple(got.shape) == (wl.B, wl.S, wl.H)
+    assert np.array_equal(got.cpu().numpy(), run_encoder(w, layers=2))
+    _check(got.cpu().numpy(), _oracle(w, layers=2), w["mask"], dtype)
 
 
 def test_empty_batch_of_tokens_and_holes():
