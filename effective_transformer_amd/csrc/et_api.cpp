@@ -18,6 +18,11 @@
 
 namespace et {
 
+namespace {
+// A launcher cannot return a status; a failed attribute call is kept here until the entry point checks its launches.
+thread_local hipError_t tls_attr_error = hipSuccess;
+}  // namespace
+
 void allow_dynamic_lds(const void* kernel, int bytes) {
   static std::mutex mu;
   static std::vector<std::pair<const void*, int>> done;      // (kernel, device) pairs already raised
@@ -26,8 +31,18 @@ void allow_dynamic_lds(const void* kernel, int bytes) {
   std::lock_guard<std::mutex> lock(mu);
   for (const auto& e : done)
     if (e.first == kernel && e.second == dev) return;
-  (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  const hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (err != hipSuccess) {
+    tls_attr_error = err;          // reported as ET_RUNTIME_ERROR by the entry point; tried again on the next call
+    return;
+  }
   if (dev >= 0) done.emplace_back(kernel, dev);
+}
+
+hipError_t take_attribute_error() {
+  const hipError_t e = tls_attr_error;
+  tls_attr_error = hipSuccess;
+  return e;
 }
 
 }  // namespace et
@@ -60,6 +75,11 @@ et_status check_hip(et_handle h, hipError_t e, const char* what, const char* fil
 }
 
 et_status check_launch(et_handle h, const char* what) {
+  const hipError_t attr = et::take_attribute_error();
+  if (attr != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(h, ET_RUNTIME_ERROR, std::string(what) + ": raising the kernel's LDS limit failed: " + hipGetErrorString(attr));
+  }
   hipError_t e = hipGetLastError();
   if (e == hipSuccess) return ET_OK;
   return fail(h, ET_LAUNCH_FAILURE, std::string(what) + ": " + hipGetErrorString(e));
@@ -118,6 +138,12 @@ struct Entry {
 et_status dims_ok(et_handle h, int B, int S, int heads, int d) {
   ET_REQUIRE(h, B >= 1 && S >= 1 && heads >= 1 && d >= 1, "batch_size, seq_len, head_num, size_per_head must be >= 1");
   ET_REQUIRE(h, (long)B * S < (1L << 30), "batch_size * seq_len too large");
+  return ET_OK;
+}
+
+// the attention kernels put the sequence on a grid dimension that holds 65535 entries
+et_status batch_fits_grid(et_handle h, int B) {
+  if (B > 65535) return fail(h, ET_UNSUPPORTED, "batch_size above 65535 is not supported by the attention kernels");
   return ET_OK;
 }
 
@@ -307,6 +333,7 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   const LayerWs ws = layer_ws(dtype, B, S, head_num, size_per_head);
   if (workspace_bytes < ws.total) return fail(h, ET_WORKSPACE_TOO_SMALL, "et_layer needs et_layer_workspace_bytes(...)");
   const et::DType dt = to_dt(dtype);
+  if ((s = batch_fits_grid(h, B)) != ET_OK) return s;
   if (!et::attention_supported(dt, S, size_per_head))
     return fail(h, ET_UNSUPPORTED, "attention kernels support size_per_head == 64 and seq_len <= 512");
   if (!et::gemm_supported(dt, H, H, 3) || !et::gemm_supported(dt, F, H, 1) || !et::gemm_supported(dt, H, F, 1))
@@ -583,6 +610,7 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
   ET_REQUIRE(h, workspace != nullptr, "null workspace");
   if (workspace_bytes < et_seq_workspace_bytes(batch_size))
     return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
+  if ((s = batch_fits_grid(h, batch_size)) != ET_OK) return s;
   if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
     return fail(h, ET_UNSUPPORTED, "attention kernels support size_per_head == 64 and seq_len <= 512");
   if (qkv_layout == 1 && ((size_t)packed_ld * et::elem_size(to_dt(dtype))) % 16 != 0)

@@ -15,6 +15,8 @@ inline size_t elem_size(DType t) { return t == DType::F32 ? 4 : 2; }
 // Kernels that need more than 64 KB of dynamic LDS raise the limit once per (kernel, device): the attribute belongs
 // to the device a module is loaded on, and a process may hold handles on several GPUs.  (et_api.cpp)
 void allow_dynamic_lds(const void* kernel, int bytes);
+// The error of a failed allow_dynamic_lds on this thread since the last call (hipSuccess if none); clears it.
+hipError_t take_attribute_error();
 
 // ---- input_output.hip --------------------------------------------------------------------
 // Number of int32 words of scratch the scan needs for `length` elements.
