@@ -47,6 +47,7 @@ def test_sweep_tables_are_the_published_ones():
 def _run_benchmark(capsys, precision):
     args = benchmark.build_parser().parse_args(["-p", precision, "-b", "8", "-m", "32", "-a", "20", "--iters", "4",
                                                 "--warmup", "2"])
+    capsys.readouterr()                                  # drop what the test itself printed
     benchmark.main(args)
     return capsys.readouterr().out
 
@@ -73,6 +74,7 @@ def test_benchmark_prints_the_reference_lines(capsys, precision, tol):
 def test_sweep_prints_one_row_per_published_row(capsys):
     print("sample sweep", flush=True)
     args = sweep.build_parser().parse_args(["--iters", "3", "--precision", "fp16", "--max-batch", "100"])
+    capsys.readouterr()
     sweep.main(args)
     rows = [l for l in capsys.readouterr().out.splitlines() if l.startswith("| fp16")]
     assert len(rows) == 2
