@@ -59,6 +59,7 @@ SIGNATURES = {
     "et_layer_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "et_seq_workspace_bytes": (_sz, [_i]),
     "et_input": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp, _ip]),
+    "et_input_static": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "et_embedding_input": (_i, [_vp, _i, C.POINTER(EmbeddingWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                                 _vp, _sz, _vp, _ip]),
     "et_layer": (_i, [_vp, _i, C.POINTER(LayerWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,

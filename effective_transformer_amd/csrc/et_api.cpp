@@ -47,6 +47,34 @@ hipError_t take_attribute_error() {
 
 }  // namespace et
 
+namespace {
+
+// Scratch of et_input_static: the tile totals of the mask scan (one int32 per tile of 1024 positions) for up to
+// kStaticMaxPositions positions.  Every GPU the library runs on holds its own copy of the array until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use is looked
+// up once per device (et_create) and kept in static_scratch_ptr.
+constexpr int kStaticScratchWords = 1024;
+constexpr int kStaticMaxPositions = 1024 * 1024;
+static __device__ __align__(256) int32_t scratch[kStaticScratchWords];
+
+constexpr int kMaxDevices = 64;
+std::mutex static_scratch_mu;
+int32_t* static_scratch_ptr[kMaxDevices] = {};
+
+// Looks up this device's copy of `scratch` (the device must be current).  Called by et_create.
+hipError_t resolve_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(static_scratch_mu);
+  if (static_scratch_ptr[device]) return hipSuccess;
+  void* p = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess) return e;
+  static_scratch_ptr[device] = static_cast<int32_t*>(p);
+  return hipSuccess;
+}
+
+}  // namespace
+
 struct et_context {
   int device = 0;
   std::mutex mu;
@@ -183,6 +211,18 @@ et_status et_create(et_handle* out, int device) {
   if (e != hipSuccess) return fail(nullptr, ET_RUNTIME_ERROR, std::string("hipGetDeviceCount: ") + hipGetErrorString(e));
   if (device < 0 || device >= count) return fail(nullptr, ET_INVALID_ARGUMENT, "no such device");
   if (!et_device_ok(device)) return fail(nullptr, ET_UNSUPPORTED, "device is not gfx950; the kernels are built for MI355X only");
+  {
+    // the address of the static scratch array on this device (et_input_static), looked up with the device current
+    int prev = 0;
+    e = hipGetDevice(&prev);
+    if (e == hipSuccess) e = hipSetDevice(device);
+    if (e == hipSuccess) {
+      e = resolve_static_scratch(device);
+      (void)hipSetDevice(prev);
+    }
+    if (e != hipSuccess)
+      return fail(nullptr, ET_RUNTIME_ERROR, std::string("static scratch lookup: ") + hipGetErrorString(e));
+  }
   et_context* c = new (std::nothrow) et_context();
   if (!c) return fail(nullptr, ET_RUNTIME_ERROR, "out of host memory");
   c->device = device;
@@ -242,6 +282,36 @@ et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const i
     ET_HIP(h, hipStreamSynchronize(st));
   }
   return ET_OK;
+}
+
+et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask, void* to_tensor,
+                          int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx, int batch_size,
+                          int seq_len, int head_num, int size_per_head, void* stream) {
+  Entry entry(h);
+  et_status s = entry.status;
+  if (s != ET_OK) return s;
+  ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
+  if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
+  ET_REQUIRE(h, from_tensor && mask && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
+  if ((long)batch_size * seq_len > kStaticMaxPositions ||
+      et::scan_scratch_words(batch_size * seq_len) > (size_t)kStaticScratchWords)
+    return fail(h, ET_UNSUPPORTED,
+                "et_input_static holds scratch for batch_size * seq_len <= 1048576 positions; larger batches go "
+                "through et_input with a caller workspace");
+  const size_t row_bytes = (size_t)head_num * size_per_head * et::elem_size(to_dt(dtype));
+  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
+  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+    return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
+  int32_t* scratch_dev = h->device < kMaxDevices ? static_scratch_ptr[h->device] : nullptr;
+  if (!scratch_dev) return fail(h, ET_RUNTIME_ERROR, "no static scratch on this device");
+  hipStream_t st = (hipStream_t)stream;
+  // the scan writes every tile total it later reads, so nothing of the previous call's contents has to be cleared
+  et::launch_scan_index(mask, batch_size * seq_len, nullptr, batch_idx, word_idx, valid_word_num_dev, seq_len,
+                        scratch_dev, st);
+  if ((s = check_launch(h, "mask scan")) != ET_OK) return s;
+  et::launch_compress_rows(from_tensor, to_tensor, batch_idx, word_idx, valid_word_num_dev, nullptr, nullptr,
+                           batch_size, seq_len, (int)row_bytes, st);
+  return check_launch(h, "compress");
 }
 
 et_status et_embedding_input(et_handle h, et_dtype dtype, const et_embedding_weights* emb, const int32_t* input_ids,

@@ -98,6 +98,17 @@ et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const i
                    int batch_size, int seq_len, int head_num, int size_per_head,
                    void* workspace, size_t workspace_bytes, void* stream, int32_t* valid_word_num_host);
 
+/* et_input for callers that cannot allocate device memory or hand over a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels, same
+ * outputs as et_input bit for bit; the scan's scratch (one int32 per 1024 mask positions) lives in a 4 KB array
+ * inside the library's device image, one copy per GPU for the life of the process, so the call takes no workspace and
+ * allocates nothing.  Limit: batch_size * seq_len <= 1048576 positions (ET_UNSUPPORTED beyond; use et_input).  Never
+ * synchronises (no host count).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (different streams or handles) race; calls ordered on one stream are safe. */
+et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask,
+                          void* to_tensor, int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx,
+                          int batch_size, int seq_len, int head_num, int size_per_head, void* stream);
+
 /* EffectiveTransformerOpFunctor::Compute, tf_op/bert_transformer_op.cu.cc:33-260
  * (op registered at tf_op/bert_transformer_op.cc:44-77): one encoder layer on packed tokens.
  *   from_tensor, to_tensor [T,H] packed; attr_mask [B,S,S] of dtype (1 = attend);
