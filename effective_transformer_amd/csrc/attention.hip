@@ -82,10 +82,10 @@ __global__ __launch_bounds__(kPadThreads) void qkv_bias_pad_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// stand-alone softmax: one wavefront per (b, head, q) row, up to 512 keys.
+// stand-alone softmax: one wavefront per (b, head, q) row, up to 1024 keys.
 // ------------------------------------------------------------------------------------------
 constexpr int kSmThreads = 256;
-constexpr int kSmMaxIters = 8;
+constexpr int kSmMaxIters = 16;
 
 template <typename T>
 __global__ __launch_bounds__(kSmThreads) void softmax_kernel(T* __restrict__ qk, const T* __restrict__ attr_mask,
@@ -98,7 +98,8 @@ __global__ __launch_bounds__(kSmThreads) void softmax_kernel(T* __restrict__ qk,
   T* x = qk + (size_t)row * seq_len;
   const T* mk = attr_mask + ((size_t)b * seq_len + q) * seq_len;
   float t[kSmMaxIters];
-  float mx = 0.f;                         // the maximum is clamped below at 0
+  // the maximum is clamped below at 0, except at 1024 keys, where the reference's max reduction has no idle lane
+  float mx = seq_len < 1024 ? 0.f : -INFINITY;
 #pragma unroll
   for (int i = 0; i < kSmMaxIters; ++i) {
     const int k = lane + i * kWave;
@@ -827,11 +828,139 @@ void attention_long_launch(const void* q, const void* k, const void* v, int layo
                                              (T*)dst, seq_start, word_idx, seq_len, heads, scaler);
 }
 
+// ------------------------------------------------------------------------------------------
+// fused attention for every shape the MFMA kernels above are not built for: size_per_head other than 64 (any
+// multiple of 16 bytes up to 256 elements) and 512 < seq_len <= 1024.  One wavefront per (query, head): the lanes
+// split the keys for the scores (full dot products in float, rounded to the element type as the reference stores
+// them), the softmax runs on wave reductions, then the lanes split the features for P.V, skipping keys whose
+// probability is 0.  Same arithmetic and rounding points as the other kernels; at seq_len = 1024 the reference's block
+// of 1024 threads leaves no idle lane in its max reduction, so the clamp of the maximum at 0 disappears there
+// (cuda/attention.cu:77-95, 267-270, 345-356: below 1024 the filler -1e-20 of the out-of-range threads acts as the clamp).
+// ------------------------------------------------------------------------------------------
+constexpr int kGenMaxSeq = 1024;
+constexpr int kGenMaxD = 256;
+
+template <typename T>
+__global__ __launch_bounds__(kAttnThreads) void attention_generic_kernel(
+    const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
+    const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ word_idx, int seq_len, int heads, int d, float scaler) {
+  using C = Chunk16<T>;
+  using V16 = typename C::vec;
+  constexpr int kPerLane = kGenMaxSeq / kWave;             // keys per lane
+  __shared__ int tok_of_pos[kGenMaxSeq];
+  __shared__ float prob[kAttnWaves][kGenMaxSeq];
+  __shared__ float qrow[kAttnWaves][kGenMaxD];
+
+  const int b = blockIdx.z, head = blockIdx.y;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  const int len = t1 - t0;
+  if (len <= 0) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int H = heads * d;
+  for (int i = threadIdx.x; i < seq_len; i += kAttnThreads) tok_of_pos[i] = -1;
+  __syncthreads();
+  for (int tt = threadIdx.x; tt < len; tt += kAttnThreads) {
+    const int pos = word_idx[t0 + tt];
+    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = t0 + tt;
+  }
+  __syncthreads();
+  const int q = blockIdx.x * kAttnWaves + wave;            // this wavefront's query position
+  if (q >= seq_len) return;
+  const int tq = tok_of_pos[q];
+  if (tq < 0) return;                                      // no token: the reference drops this row
+  auto src_off = [&](int t, int pos) -> size_t {
+    return layout == 1 ? (size_t)t * packed_ld + head * d : (((size_t)b * heads + head) * seq_len + pos) * d;
+  };
+  for (int j = lane; j < d; j += kWave) qrow[wave][j] = (float)q_src[src_off(tq, q) + j];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // ---- scores of the lane's keys: key = lane + 64 i --------------------------------------------------------
+  const T* mrow = attr_mask + ((size_t)b * seq_len + q) * seq_len;
+  float t[kPerLane];
+  float mx = seq_len < kGenMaxSeq ? 0.f : -INFINITY;       // the clamp at 0 holds below 1024 keys
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) {
+    const int key = lane + i * kWave;
+    t[i] = -INFINITY;
+    if (key < seq_len) {
+      const int tk = tok_of_pos[key];
+      float dot = 0.f;
+      if (tk >= 0) {
+        const T* krow = k_src + src_off(tk, key);
+        for (int c = 0; c < d; c += C::kElems) {
+          const V16 kv = *reinterpret_cast<const V16*>(krow + c);
+#pragma unroll
+          for (int j = 0; j < C::kElems; ++j) dot += qrow[wave][c + j] * (float)kv[j];
+        }
+      }
+      const float sc = (float)(T)dot;                      // the score is stored in the element type
+      t[i] = sc * scaler + (1.0f - (float)mrow[key]) * -10000.0f;
+      mx = fmaxf(mx, t[i]);
+    }
+  }
+  mx = wave_max(mx) * kLog2e;
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) {
+    t[i] = __builtin_amdgcn_exp2f(t[i] * kLog2e - mx);     // exp2(-inf) = 0 for absent keys
+    sum += t[i];
+  }
+  sum = wave_sum(sum) + 1e-6f;
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) {
+    const int key = lane + i * kWave;
+    if (key < seq_len) prob[wave][key] = (float)(T)(t[i] * inv);     // the probability is stored in the element type
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // ---- P.V: feature = lane + 64 i ------------------------------------------------------------------------------
+  constexpr int kFeat = kGenMaxD / kWave;
+  float acc[kFeat];
+#pragma unroll
+  for (int i = 0; i < kFeat; ++i) acc[i] = 0.f;
+  for (int key = 0; key < seq_len; ++key) {
+    const int tk = tok_of_pos[key];
+    const float pk = prob[wave][key];
+    if (tk < 0 || pk == 0.f) continue;                     // wave-uniform: a zero value or a zero weight
+    const T* vrow = v_src + src_off(tk, key);
+#pragma unroll
+    for (int i = 0; i < kFeat; ++i) {
+      const int j = lane + i * kWave;
+      if (j < d) acc[i] += pk * (float)vrow[j];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kFeat; ++i) {
+    const int j = lane + i * kWave;
+    if (j < d) dst[(size_t)tq * H + head * d + j] = (T)acc[i];
+  }
+}
+
+template <typename T>
+void attention_generic_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
+                              void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len,
+                              int heads, int d, float scaler, hipStream_t stream) {
+  dim3 grid((seq_len + kAttnWaves - 1) / kAttnWaves, heads, batch);
+  attention_generic_kernel<T><<<grid, kAttnThreads, 0, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
+                                                                 (const T*)attr_mask, (T*)dst, seq_start, word_idx, seq_len,
+                                                                 heads, d, scaler);
+}
+
 template <typename T>
 void attention_dispatch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                         void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
-                        float scaler, hipStream_t stream) {
-  if (seq_len > 256)
+                        int d, float scaler, hipStream_t stream) {
+  if (d != kD || seq_len > 512)
+    attention_generic_launch<T>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads, d,
+                                scaler, stream);
+  else if (seq_len > 256)
     attention_long_launch<T, 32>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
                                  scaler, stream);
   else if (seq_len > 128)
@@ -895,20 +1024,19 @@ void launch_transpose_rm_padding(DType t, const void* src, void* dst, const int3
 }
 
 bool attention_supported(DType t, int seq_len, int d) {
-  (void)t;
-  return d == kD && seq_len >= 1 && seq_len <= 512;
+  // rows of a head are moved in 16-byte pieces
+  return d >= 1 && d <= kGenMaxD && ((size_t)d * elem_size(t)) % 16 == 0 && seq_len >= 1 && seq_len <= kGenMaxSeq;
 }
 
 void launch_attention(DType t, const void* q, const void* k, const void* v, int layout, int packed_ld,
                       const void* attr_mask, void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch,
                       int seq_len, int heads, int d, float scaler, hipStream_t stream) {
-  (void)d;
   if (t == DType::F32)
-    attention_dispatch<float>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+    attention_dispatch<float>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads, d,
                               scaler, stream);
   else
     attention_dispatch<_Float16>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len,
-                                 heads, scaler, stream);
+                                 heads, d, scaler, stream);
 }
 
 }  // namespace et

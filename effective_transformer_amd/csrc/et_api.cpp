@@ -405,7 +405,7 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   const et::DType dt = to_dt(dtype);
   if ((s = batch_fits_grid(h, B)) != ET_OK) return s;
   if (!et::attention_supported(dt, S, size_per_head))
-    return fail(h, ET_UNSUPPORTED, "attention kernels support size_per_head == 64 and seq_len <= 512");
+    return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 in multiples of 16 bytes and seq_len <= 1024");
   if (!et::gemm_supported(dt, H, H, 3) || !et::gemm_supported(dt, F, H, 1) || !et::gemm_supported(dt, H, F, 1))
     return fail(h, ET_UNSUPPORTED, "hidden size not supported by the GEMM kernels");
   if ((uint64_t)B * S * F * et::elem_size(dt) > 0xffffffffull)
@@ -644,7 +644,7 @@ et_status et_softmax(et_handle h, et_dtype dtype, void* qk_buf, const void* attr
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, 1)) != ET_OK) return s;
   ET_REQUIRE(h, qk_buf && attr_mask, "null tensor pointer");
-  if (seq_len > 512) return fail(h, ET_UNSUPPORTED, "softmax kernel supports seq_len <= 512");
+  if (seq_len > 1024) return fail(h, ET_UNSUPPORTED, "softmax kernel supports seq_len <= 1024");
   et::launch_softmax(to_dt(dtype), qk_buf, attr_mask, batch_size, head_num, seq_len, scaler, (hipStream_t)stream);
   return check_launch(h, "softmax");
 }
@@ -682,7 +682,7 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
     return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
   if ((s = batch_fits_grid(h, batch_size)) != ET_OK) return s;
   if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
-    return fail(h, ET_UNSUPPORTED, "attention kernels support size_per_head == 64 and seq_len <= 512");
+    return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 in multiples of 16 bytes and seq_len <= 1024");
   if (qkv_layout == 1 && ((size_t)packed_ld * et::elem_size(to_dt(dtype))) % 16 != 0)
     return fail(h, ET_UNSUPPORTED, "packed_ld bytes must be a multiple of 16");
   hipStream_t st = (hipStream_t)stream;

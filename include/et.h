@@ -117,7 +117,8 @@ et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, 
  * then sized for B*S rows and every kernel bounds itself by *valid_word_num_dev, so the call
  * never blocks the host (the reference copies T back every layer, :99-101).
  * from_seq_len must equal to_seq_len (tf_op/bert_transformer_op.cc:130-131).  `out` must not
- * alias from_tensor/to_tensor. */
+ * alias from_tensor/to_tensor.  Shapes: seq_len <= 1024, batch_size <= 65535, size_per_head <= 256 (see et_attention),
+ * hidden size a multiple of 32 (fp16) or 16 (fp32). */
 et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
                    const void* from_tensor, const void* to_tensor, const void* attr_mask,
                    const int32_t* valid_word_num_dev, const int32_t* batch_idx, const int32_t* word_idx,
@@ -242,7 +243,9 @@ et_status et_add_qkv_bias_padding(et_handle h, et_dtype dtype,
                                   void* workspace, size_t workspace_bytes, void* stream);
 
 /* softmax_kernel_kernelLauncher, cuda/attention.h:37-42 (cuda/attention.cu:249-382): in-place
- * masked, scaled softmax of qk_buf [B,heads,S,S] with attr_mask [B,S,S]. */
+ * masked, scaled softmax of qk_buf [B,heads,S,S] with attr_mask [B,S,S], S <= 1024 (the reach of the reference's
+ * launcher, :345-356).  As in the reference the row maximum is clamped below at 0 for S < 1024 and is the true maximum
+ * at S = 1024 (:77-95, 267-270). */
 et_status et_softmax(et_handle h, et_dtype dtype, void* qk_buf, const void* attr_mask,
                      int batch_size, int head_num, int seq_len, float scaler, void* stream);
 
@@ -258,7 +261,9 @@ et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, 
  *   qkv_layout 0: q/k/v are the padded [B,heads,S,d] buffers add_QKV_bias_padding writes;
  *   qkv_layout 1: q/k/v point into packed token-major rows (row t, column head*d + j) with row
  *                 stride `packed_ld` elements (bias already added).
- *   dst packed [T,heads*d].  workspace: et_seq_workspace_bytes(B). */
+ *   dst packed [T,heads*d].  workspace: et_seq_workspace_bytes(B).
+ * seq_len <= 1024; size_per_head <= 256 with head rows of whole 16-byte pieces.  size_per_head = 64 with
+ * seq_len <= 512 runs the MFMA kernels, every other shape a slower general kernel with the same arithmetic. */
 et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v, int qkv_layout,
                        int packed_ld, const void* attr_mask, void* dst,
                        const int32_t* valid_word_num_dev, int batch_size, int seq_len,

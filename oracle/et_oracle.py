@@ -243,12 +243,15 @@ def softmax(qk, attr_mask, scaler: float, dtype: str):
       p = e / (sum e + 1e-6).
     The clamp of the maximum at 0 comes from the second stage of blockReduceMax
     (cuda/attention.cu:91-92), which feeds 0 for idle lanes whenever the block has
-    fewer than 32 warps, i.e. for every S <= 512."""
+    fewer than 32 warps, i.e. for every S <= 512.  For 512 < S < 1024 the block has 1024
+    threads (:345-356) and the threads beyond S feed -1e-20 into the reduction
+    (:267-270), which in float acts exactly like the clamp at 0 (t - (-1e-20) == t);
+    only S = 1024 has neither and uses the true maximum."""
     S = qk.shape[-1]
     t = (qk.astype(np.float32) * np.float32(scaler)).astype(np.float32)
     mv = ((np.float32(1.0) - attr_mask.astype(np.float32)) * np.float32(-10000.0)).astype(np.float32)
     t = (t + mv[:, None, :, :]).astype(np.float32)
-    m = np.maximum(t.max(axis=-1, keepdims=True), np.float32(0.0)) if S <= 512 else t.max(axis=-1, keepdims=True)
+    m = np.maximum(t.max(axis=-1, keepdims=True), np.float32(0.0)) if S < 1024 else t.max(axis=-1, keepdims=True)
     e = np.exp((t - m).astype(np.float64))
     e = np.where((t - m) < -103.0, 0.0, e)        # float32 exp underflows to 0 below ~-103.97
     p = e / (e.sum(axis=-1, keepdims=True) + 1e-6)

@@ -252,8 +252,8 @@ def test_error_paths():
     with pytest.raises(_lib.EtError) as e:       # from_seq_len != to_seq_len
         ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S + 1, wl.heads, wl.d)
     assert e.value.status == 1 and "from_seq_len == to_seq_len" in str(e.value)
-    with pytest.raises(_lib.EtError) as e:       # size_per_head the attention kernel is not built for
-        ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S, wl.heads * 2, wl.d // 2)
+    with pytest.raises(_lib.EtError) as e:       # a head row that is not a whole number of 16-byte pieces
+        ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S, wl.heads * 32, wl.d // 32)
     assert e.value.status == 3
     out = torch.empty_like(to)
     st = lib.et_layer(h, 0, C.byref(lw.struct), to.data_ptr(), to.data_ptr(), attr.data_ptr(), vwn.data_ptr(),
@@ -281,6 +281,22 @@ def test_long_sequences_layer_against_oracle(dtype):
     for _ in range(2):
         weights.extend(o.make_layer_weights(wl, rng, True))
     w = dict(wl=wl, lens=lens, mask=mask, attr_mask=attr, x=x, weights=weights)
+    got = run_encoder(w)
+    _check(got, _oracle(w), mask, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("B,S,heads,d", [(4, 48, 4, 32), (3, 40, 2, 128), (2, 600, 2, 64), (1, 1024, 1, 64), (2, 520, 4, 32)])
+def test_other_head_sizes_and_sequences_beyond_512(dtype, B, S, heads, d):
+    """The reference op takes any size_per_head (tf_op/bert_transformer_op.cc:53-57) and sequences up to the 1024 keys
+    its softmax launcher covers (cuda/attention.cu:345-356): one layer against the oracle."""
+    print("encoder other shapes", dtype, B, S, heads, d, flush=True)
+    wl = o.Workload("odd", 500 + S + d, dtype, 1, B, S, heads, d, 4 * heads * d, max(1, S // 3), S + 1)
+    rng = np.random.RandomState(wl.seed)
+    lens, mask, attr = o.make_masks(wl, rng)
+    lens[0] = S; mask[0] = 1; attr[0] = 1                   # one sequence of full length
+    x = o.rnd(rng.randn(B, S, wl.H), dtype)
+    w = dict(wl=wl, lens=lens, mask=mask, attr_mask=o.rnd(attr, dtype), x=x, weights=o.make_layer_weights(wl, rng, True))
     got = run_encoder(w)
     _check(got, _oracle(w), mask, dtype)
 

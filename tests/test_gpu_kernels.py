@@ -174,9 +174,8 @@ def test_add_bias_input_layernorm(k, dtype, m, n):
 
 # ---------------------------------------------------------------- attention side ---
 
-def _attn_problem(seed, B, S, heads, dtype, holes=False, weird_mask=False):
+def _attn_problem(seed, B, S, heads, dtype, holes=False, weird_mask=False, d=64):
     rng = np.random.RandomState(seed)
-    d = 64
     if holes:
         mask = (rng.random_sample((B, S)) < 0.6).astype(np.int32)
         mask[0] = 0                                  # an empty sequence
@@ -221,7 +220,7 @@ def test_qkv_bias_padding_and_unpad(k, dtype, holes):
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
-@pytest.mark.parametrize("S", [1, 7, 32, 64, 100, 128, 300])
+@pytest.mark.parametrize("S", [1, 7, 32, 64, 100, 128, 300, 513, 600, 1024])
 def test_softmax(k, dtype, S):
     rng = np.random.RandomState(S)
     B, heads = 3, 2
@@ -235,7 +234,10 @@ def test_softmax(k, dtype, S):
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-7)
     else:
         assert_half_close(got, want, ulps=1.0, frac=0.02, what="softmax")
-    assert np.all(got[0, :, 0, :] == 0)                      # fully masked row -> zeros (maximum clamped at 0)
+    if S < 1024:
+        assert np.all(got[0, :, 0, :] == 0)                  # fully masked row -> zeros (maximum clamped at 0)
+    else:
+        assert np.all(got[0, :, 0, :] > 0)                   # 1024 keys: no clamp, a fully masked row stays a distribution
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
@@ -267,6 +269,38 @@ def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
         np.testing.assert_allclose(got0[:T], want, rtol=1e-4, atol=2e-5)
     else:
         # fp32 accumulation vs the oracle's exact sums, three roundings to half on the way
+        np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("S,d,holes,weird", [(40, 32, False, False), (70, 128, True, True), (33, 8, True, False),
+                                             (16, 256, False, True), (600, 64, False, False), (513, 64, True, True),
+                                             (1024, 64, False, True), (1000, 32, True, False)])
+def test_fused_attention_other_head_sizes_and_long_sequences(k, dtype, S, d, holes, weird):
+    """size_per_head other than 64 (the reference op takes any, tf_op/bert_transformer_op.cc:53-57) and 512 < seq_len <= 1024
+    (its softmax launcher's last branch, cuda/attention.cu:345-356; no clamp of the maximum at 1024 keys)."""
+    print("attention generic", dtype, S, d, holes, weird, flush=True)
+    if dtype == "fp32" and d == 8:
+        d = 12                                             # rows move in 16-byte pieces
+    B, heads = 3, 2
+    p = _attn_problem(S + d, B, S, heads, dtype, holes=holes, weird_mask=weird, d=d)
+    bi, wi, vwn = _idx_dev(p)
+    T = p["T"]
+    H = heads * d
+    qp, kp, vp = o.add_qkv_bias_padding(p["q"], p["bq"], p["k"], p["bk"], p["v"], p["bv"], T, B, S, heads, d, p["bi"],
+                                        p["wi"], dtype)
+    want = o.attention(qp, kp, vp, p["attr"], T, p["bi"], p["wi"], dtype)
+    got0 = k.attention(dev(qp), dev(kp), dev(vp), 0, 0, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    add = (lambda a, b: (a.astype(np.float32) + b.astype(np.float32)).astype(np.float32)) if dtype == "fp32" else o.hadd
+    packed = np.zeros((B * S, 3 * H), o._np_dtype(dtype))
+    packed[:T, :H] = add(p["q"], p["bq"]); packed[:T, H:2 * H] = add(p["k"], p["bk"]); packed[:T, 2 * H:] = add(p["v"], p["bv"])
+    pk = dev(packed)
+    got1 = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    assert np.array_equal(got0, got1)
+    assert np.all(got0[T:] == 0)
+    if dtype == "fp32":
+        np.testing.assert_allclose(got0[:T], want, rtol=1e-4, atol=2e-5)
+    else:
         np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
 
 

@@ -178,6 +178,31 @@ def test_softmax_against_torch_and_quirks():
     np.testing.assert_allclose(p[0, 0, 0, 0], 1 / (1 + math.exp(-10) + 1e-6), rtol=1e-6)
 
 
+def test_softmax_clamp_rule_by_block_size():
+    """Which rows see the clamp of the maximum follows from the launch geometry (cuda/attention.cu:345-356) and the
+    two fillers of the reduction (:91-92 idle lanes give 0, :267-270 out-of-range threads give -1e-20): up to 1023 keys a
+    fully masked row is all zeros (every term exp(-10000 - 0) underflows), at exactly 1024 keys nothing clamps and the
+    row is uniform.  Brute force per row in float64 with that rule written out."""
+    rng = np.random.RandomState(4)
+    for S in (512, 513, 600, 1023, 1024):
+        qk = (3 * rng.randn(1, 1, 2, S)).astype(np.float32)
+        mask = np.ones((1, 2, S), np.float32)
+        mask[0, 1] = 0                                                # second query row fully masked
+        got = o.softmax(qk, mask, 0.125, "fp32")      # a [2,S] slab of query rows is enough for the row-wise arithmetic
+        t0 = qk[0, 0, 0].astype(np.float64) * 0.125
+        m0 = max(t0.max(), 0.0) if S < 1024 else t0.max()
+        e0 = np.exp(t0 - m0)
+        np.testing.assert_allclose(got[0, 0, 0], e0 / (e0.sum() + 1e-6), rtol=2e-6)
+        if S < 1024:
+            assert np.all(got[0, 0, 1] == 0)
+        else:
+            # the kernel adds the -10000 in float (cuda/attention.cu:262-265): at that magnitude a float step is 1e-3
+            t1 = ((qk[0, 0, 1] * np.float32(0.125)).astype(np.float32) + np.float32(-10000.0)).astype(np.float64)
+            e1 = np.exp(t1 - t1.max())
+            np.testing.assert_allclose(got[0, 0, 1], e1 / (e1.sum() + 1e-6), rtol=1e-4)
+            assert got[0, 0, 1].min() > 0
+
+
 def test_qkv_pad_and_unpad_brute_force():
     rng = np.random.RandomState(3)
     B, S, heads, d = 3, 5, 2, 4
