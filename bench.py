@@ -18,17 +18,76 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (FETCH_SIZE scaled by 2.0, the factor a
-# plain device copy of known size shows in the same run); cfg3 shapes.  (read + write) in bytes.
-MEASURED_TRAFFIC = {
-    ("cfg3", "gemm_ffn_up"): (377.2 + 236.7) * (1 << 20),
-    ("cfg3", "gemm_ffn_down"): (328.0 + 59.3) * (1 << 20),
-    ("cfg3", "gemm_qkv"): (241.0 + 177.7) * (1 << 20),
-    ("cfg3", "gemm_attn_out"): (86.0 + 59.3) * (1 << 20),
-    ("cfg3", "bias_gelu"): (236.8 + 236.7) * (1 << 20),
-    ("cfg3", "bias_residual_layernorm"): (118.4 + 59.2) * (1 << 20),
-    ("cfg3", "attention"): (202.2 + 59.2) * (1 << 20),
-}
+# HBM bytes per launch come from profiles/hbm_traffic.json when it holds an entry for the workload and kernel: two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch) folded in by
+# `bench.py --fold-traffic`, each counter scaled by what it reads for the plain device copy of --calibrate-copy.  The
+# file names the commit it was measured on; without an entry `traffic` is null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+# kernel name in the counter files -> key in `kernels`, for the kernels one name identifies (the FFN-up projection is the
+# only launch of the GELU instance of the large-M GEMM; the other three projections share one instance)
+TRAFFIC_KERNELS = (("gemm_f16_pair_kernel<true>", "gemm_ffn_up"), ("gemm_f16_pair_kernelILb1", "gemm_ffn_up"),
+                   ("attention_kernel", "attention"), ("attention_long_kernel", "attention"),
+                   ("bias_residual_layernorm_kernel", "bias_residual_layernorm"), ("bias_gelu_kernel", "bias_gelu"),
+                   ("restore_rows_kernel", "output_restore"))
+COPY_BYTES = 256 << 20
+
+
+def measured_traffic(workload, kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            d = json.load(f)
+        e = d["workloads"][workload][kernel]
+        return {"bytes": e["read_bytes"] + e["write_bytes"], "read_bytes": e["read_bytes"], "write_bytes": e["write_bytes"],
+                "source": "profiles/hbm_traffic.json", "measured_on_commit": d["workloads"][workload].get("commit")}
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def fold_traffic(workload, fetch_csv, write_csv, commit, command):
+    """Folds two counter files (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --calibrate-copy`) into
+    profiles/hbm_traffic.json."""
+    import collections
+    import csv
+
+    def load(path):
+        agg = collections.defaultdict(list)
+        for r in csv.DictReader(open(path)):
+            agg[r["Kernel_Name"]].append(float(r["Counter_Value"]) * 1024.0)      # KiB per dispatch
+        return agg
+
+    fe, wr = load(fetch_csv), load(write_csv)
+
+    def mean_of(agg, sub):
+        v = [x for k, vals in agg.items() if sub in k for x in vals]
+        return (sum(v) / len(v), len(v)) if v else (None, 0)
+
+    # the copy of --calibrate-copy is the largest device copy of the run
+    cf = max([x for k, vals in fe.items() if "copyBuffer" in k for x in vals], default=0)
+    cw = max([x for k, vals in wr.items() if "copyBuffer" in k for x in vals], default=0)
+    if not cf or not cw:
+        sys.exit("no device copy in the counter files: run bench.py with --calibrate-copy under rocprofv3")
+    scale_f, scale_w = COPY_BYTES / cf, COPY_BYTES / cw
+    entry = {"commit": commit, "command": command,
+             "scale": {"FETCH_SIZE": round(scale_f, 3), "WRITE_SIZE": round(scale_w, 3),
+                       "from": "device copy of %d bytes in the same runs" % COPY_BYTES}}
+    for sub, key in TRAFFIC_KERNELS:
+        f, n = mean_of(fe, sub)
+        w, _ = mean_of(wr, sub)
+        if f is None or w is None or key in entry:
+            continue
+        entry[key] = {"read_bytes": round(f * scale_f), "write_bytes": round(w * scale_w), "dispatches": n}
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            d = json.load(fh)
+    except (OSError, ValueError):
+        d = {"workloads": {}}
+    d["workloads"][workload] = entry
+    with open(TRAFFIC_FILE, "w") as fh:
+        json.dump(d, fh, indent=1, sort_keys=True)
+        fh.write("\n")
+    print(json.dumps(entry, indent=1))
+
+
 # ms/batch the reference publishes for the same model/batch/sequence recipe (Tesla V100, Readme.md:65-89 of the
 # reference); vs_baseline = published ms / measured ms.
 PUBLISHED_MS = {"cfg2": (8.75, "Readme.md:65"), "cfg3": (133.61, "Readme.md:80"), "cfg4": (325.37, "Readme.md:89")}
@@ -276,7 +335,15 @@ def main():
     ap.add_argument("--cpu-seqs", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--fold-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no benchmark: fold two rocprofv3 --pmc counter files into profiles/hbm_traffic.json")
+    ap.add_argument("--commit", default="unknown", help="with --fold-traffic: the commit the counters were measured on")
     a = ap.parse_args()
+    if a.fold_traffic:
+        fold_traffic(a.workload, a.fold_traffic[0], a.fold_traffic[1], a.commit,
+                     "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -d out -o fetch|write -- python3 bench.py "
+                     "--workload %s --steps 2 --warmup 1 --no-cpu --calibrate-copy" % a.workload)
+        return
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every box here has one); --gpus %d is not supported" % a.gpus)
 
@@ -311,7 +378,7 @@ def main():
     ms = s.elapsed_time(e) / a.steps
 
     if a.calibrate_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        src = torch.empty(COPY_BYTES, dtype=torch.uint8, device="cuda").fill_(1)
         dst = torch.empty_like(src)
         for _ in range(5):
             dst.copy_(src)
@@ -355,12 +422,12 @@ def main():
             roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved"], "peak": kd["peak"],
                     "unit": kd["unit"], "frac": kd["frac"], "ms": kd["ms"],
                     "measured": "HIP events around a launch loop of the kernel alone (the layer replica is host-bound at this size)",
-                    "traffic": MEASURED_TRAFFIC.get((wl.name, dom))}
+                    "traffic": measured_traffic(wl.name, dom)}
         else:
             roof = {"kernel": dom, "bound": kd["bound"], "achieved": kd["achieved_in_layer"], "peak": kd["peak"],
                     "unit": kd["unit"], "frac": kd["frac_in_layer"], "ms": kd["ms_in_layer"],
                     "measured": "HIP events around the kernel inside the layer's launch sequence, %d launches" % (4 * wl.layers),
-                    "alone": alone, "traffic": MEASURED_TRAFFIC.get((wl.name, dom))}
+                    "alone": alone, "traffic": measured_traffic(wl.name, dom)}
     cpu = None
     if not a.no_cpu:
         cpu = cpu_baseline(w, a.cpu_seqs)
