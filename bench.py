@@ -184,8 +184,9 @@ def per_kernel(wl, T, mask_np, iters=20):
     # fused attention on packed rows
     qkv = rnd(B * S, 3 * H)
     ctx = torch.empty(B * S, H, device="cuda", dtype=dt)
+    starts = ops.sequence_starts(vwn, bidx, B, S)          # one table per batch, as the encoder builds it
     ms = _time_kernel(lambda: k.attention(qkv, qkv[:, H:], qkv[:, 2 * H:], 1, 3 * H, attr, vwn, B, S, heads, d, bidx,
-                                          widx, dst=ctx), iters)
+                                          widx, dst=ctx, seq_start=starts), iters)
     lens = mask_np.sum(axis=1).astype(np.float64)
     add("attention", ms, "hbm", 4 * T * H * e + B * S * S * e + 8 * T)
     res["attention"]["valid_tflops"] = round(4 * H * float((lens ** 2).sum()) / ms / 1e9, 2)
@@ -252,6 +253,7 @@ def in_layer_kernels(wl, T, mask_np, reps=4):
     inter = torch.empty(T, F, device="cuda", dtype=dt)
     names = ("gemm_qkv", "attention", "gemm_attn_out", "bias_residual_layernorm", "gemm_ffn_up", "gemm_ffn_down",
              "bias_residual_layernorm")
+    starts = ops.sequence_starts(vwn, bidx, B, S)          # one table per batch, as the encoder builds it
 
     def layer(ev):
         cur, down = x, spare
@@ -261,7 +263,8 @@ def in_layer_kernels(wl, T, mask_np, reps=4):
             if e: e[0].record()
             f(cur, w, bias=bias["gemm_qkv"], out=qkv)
             if e: e[1].record()
-            k.attention(qkv, qkv[:, H:], qkv[:, 2 * H:], 1, 3 * H, attr, vwn, B, S, heads, d, bidx, widx, dst=ctx)
+            k.attention(qkv, qkv[:, H:], qkv[:, 2 * H:], 1, 3 * H, attr, vwn, B, S, heads, d, bidx, widx, dst=ctx,
+                        seq_start=starts)
             if e: e[2].record()
             f, w = mm["gemm_attn_out"]
             f(ctx, w, out=ao)

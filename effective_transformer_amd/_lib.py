@@ -79,6 +79,8 @@ SIGNATURES = {
     "et_softmax": (_i, [_vp, _i, _vp, _vp, _i, _i, _i, C.c_float, _vp]),
     "et_transpose_rm_padding": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "et_attention": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _sz, _vp]),
+    "et_attention_with_starts": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp,
+                                      _vp]),
     "et_gemm": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_gemm_bias_gelu": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_transpose_weight": (_i, [_vp, _i, _vp, _vp, _i, _i, _vp]),

@@ -669,6 +669,21 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
                        int packed_ld, const void* attr_mask, void* dst, const int32_t* valid_word_num_dev,
                        int batch_size, int seq_len, int head_num, int size_per_head, const int32_t* batch_idx,
                        const int32_t* word_idx, void* workspace, size_t workspace_bytes, void* stream) {
+  if (h) {
+    ET_REQUIRE(h, workspace != nullptr, "null workspace");
+    if (workspace_bytes < et_seq_workspace_bytes(batch_size))
+      return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
+  }
+  return et_attention_with_starts(h, dtype, q, k, v, qkv_layout, packed_ld, attr_mask, dst, valid_word_num_dev,
+                                  batch_size, seq_len, head_num, size_per_head, batch_idx, word_idx, nullptr,
+                                  (int32_t*)workspace, stream);
+}
+
+et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v,
+                                   int qkv_layout, int packed_ld, const void* attr_mask, void* dst,
+                                   const int32_t* valid_word_num_dev, int batch_size, int seq_len, int head_num,
+                                   int size_per_head, const int32_t* batch_idx, const int32_t* word_idx,
+                                   const int32_t* seq_start, int32_t* seq_start_scratch, void* stream) {
   Entry entry(h);
   et_status s = entry.status;
   if (s != ET_OK) return s;
@@ -677,18 +692,19 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
   ET_REQUIRE(h, q && k && v && attr_mask && dst && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
   ET_REQUIRE(h, qkv_layout == 0 || qkv_layout == 1, "qkv_layout must be 0 (padded) or 1 (packed)");
   ET_REQUIRE(h, qkv_layout == 0 || packed_ld >= head_num * size_per_head, "packed_ld smaller than the hidden size");
-  ET_REQUIRE(h, workspace != nullptr, "null workspace");
-  if (workspace_bytes < et_seq_workspace_bytes(batch_size))
-    return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
+  ET_REQUIRE(h, seq_start != nullptr || seq_start_scratch != nullptr, "null sequence start table");
   if ((s = batch_fits_grid(h, batch_size)) != ET_OK) return s;
   if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
     return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 in multiples of 16 bytes and seq_len <= 1024");
   if (qkv_layout == 1 && ((size_t)packed_ld * et::elem_size(to_dt(dtype))) % 16 != 0)
     return fail(h, ET_UNSUPPORTED, "packed_ld bytes must be a multiple of 16");
   hipStream_t st = (hipStream_t)stream;
-  et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, (int32_t*)workspace, st);
-  et::launch_attention(to_dt(dtype), q, k, v, qkv_layout, packed_ld, attr_mask, dst, (int32_t*)workspace, word_idx,
-                       batch_size, seq_len, head_num, size_per_head, softmax_scaler(dtype, size_per_head), st);
+  if (!seq_start) {
+    et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, seq_start_scratch, st);
+    seq_start = seq_start_scratch;
+  }
+  et::launch_attention(to_dt(dtype), q, k, v, qkv_layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch_size,
+                       seq_len, head_num, size_per_head, softmax_scaler(dtype, size_per_head), st);
   return check_launch(h, "attention");
 }
 

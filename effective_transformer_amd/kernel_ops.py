@@ -87,11 +87,17 @@ def transpose_rm_padding(src, valid_word_num, batch_idx, word_idx):
 
 
 def attention(q, k, v, layout: int, packed_ld: int, attr_mask, valid_word_num, B, S, heads, d, batch_idx, word_idx,
-              dst: Optional[torch.Tensor] = None):
+              dst: Optional[torch.Tensor] = None, seq_start: Optional[torch.Tensor] = None):
+    """seq_start: the table of ops.sequence_starts for this batch; the call is then the attention kernel alone."""
     lib = _lib.load()
     dev = attr_mask.device
     if dst is None:
         dst = torch.zeros(B * S, heads * d, dtype=attr_mask.dtype, device=dev)
+    if seq_start is not None:
+        _call("et_attention_with_starts", dev, _dtype_code(attr_mask.dtype), _p(q), _p(k), _p(v), layout, packed_ld,
+              _p(attr_mask), _p(dst), _p(valid_word_num), B, S, heads, d, _p(batch_idx), _p(word_idx), _p(seq_start), None,
+              _stream())
+        return dst
     ws = _workspace(dev, "seq", lib.et_seq_workspace_bytes(B))
     _call("et_attention", dev, _dtype_code(attr_mask.dtype), _p(q), _p(k), _p(v), layout, packed_ld, _p(attr_mask),
           _p(dst), _p(valid_word_num), B, S, heads, d, _p(batch_idx), _p(word_idx), _p(ws), ws.numel(), _stream())

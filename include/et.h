@@ -271,6 +271,16 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
                        const int32_t* batch_idx, const int32_t* word_idx,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* et_attention with the sequence start table of et_sequence_starts handed in (seq_start, int32[B+1]; one table serves
+ * every layer of a batch, as in et_layer_with_prepared), so that the call is the attention kernel alone.  With
+ * seq_start NULL the table is built into seq_start_scratch (int32[B+1]) first, which is what et_attention does.  No
+ * counterpart in the reference, whose attention works on padded buffers. */
+et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v,
+                                   int qkv_layout, int packed_ld, const void* attr_mask, void* dst,
+                                   const int32_t* valid_word_num_dev, int batch_size, int seq_len, int head_num,
+                                   int size_per_head, const int32_t* batch_idx, const int32_t* word_idx,
+                                   const int32_t* seq_start, int32_t* seq_start_scratch, void* stream);
+
 /* Replaces the cublasGemmEx call sites (tf_op/bert_transformer_op.cu.cc:110-141, 200-240):
  * C[m,n] = A[m,k] . B[k,n], all row-major, alpha = 1, beta = 0, fp32 accumulation, C of dtype.
  * bias (optional, [n]) is added to the rounded product (in the element type, as the reference's

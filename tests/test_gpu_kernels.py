@@ -265,6 +265,12 @@ def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
     got1 = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
     assert np.array_equal(got0, got1)
     assert np.all(got0[T:] == 0)
+    # the same call with the batch's sequence start table handed in (et_attention_with_starts)
+    from effective_transformer_amd import ops as _ops
+    starts = _ops.sequence_starts(vwn, bi, B, S)
+    got2 = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(p["attr"]), vwn, B, S, heads, d, bi, wi,
+                       seq_start=starts).cpu().numpy()
+    assert np.array_equal(got0, got2)
     if dtype == "fp32":
         np.testing.assert_allclose(got0[:T], want, rtol=1e-4, atol=2e-5)
     else:
