@@ -206,7 +206,7 @@ template <typename T, int NKT, int CPT, bool PF>
 __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
-    const int32_t* __restrict__ word_idx, int seq_len, int heads, int heads_per_wg, float scaler) {
+    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, int heads_per_wg, float scaler) {
   using Cfg = AttnCfg<T>;
   using Sm = AttnSmem<T, NKT>;
   using C = Chunk16<T>;
@@ -224,7 +224,9 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   T* Vt = reinterpret_cast<T*>(smem_raw + 2 * Sm::kQBytes);
   int* tok_of_pos = reinterpret_cast<int*>(smem_raw + 2 * Sm::kQBytes + Sm::kVtBytes);
 
-  const int b = blockIdx.y;
+  // workgroups are dealt out in the order of the table's second half: sequences of similar length side by side, the
+  // longest first
+  const int b = min(max(seq_start[batch + 1 + blockIdx.y], 0), batch - 1);
   const int h_begin = blockIdx.x * heads_per_wg;
   const int h_end = min(h_begin + heads_per_wg, heads);
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
@@ -525,8 +527,8 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
     }
   dim3 grid((heads + hpw - 1) / hpw, batch);
   kern<<<grid, kAttnThreads, Sm::kBytes, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
-                                                   (const T*)attr_mask, (T*)dst, seq_start, word_idx, seq_len, heads,
-                                                   hpw, scaler);
+                                                   (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch, seq_len,
+                                                   heads, hpw, scaler);
 }
 
 
@@ -555,7 +557,7 @@ template <typename T, int NKT>
 __global__ __launch_bounds__(kAttnThreads) void attention_long_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
-    const int32_t* __restrict__ word_idx, int seq_len, int heads, float scaler) {
+    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, float scaler) {
   using Sm = LongSmem<T>;
   using C = Chunk16<T>;
   using V16 = typename C::vec;
@@ -571,7 +573,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_long_kernel(
   T* Vs = Ks;
   int* tok_of_pos = reinterpret_cast<int*>(smem_raw + Sm::kTileBytes);
 
-  const int b = blockIdx.z, head = blockIdx.y, qblock = blockIdx.x;
+  const int b = min(max(seq_start[batch + 1 + blockIdx.z], 0), batch - 1), head = blockIdx.y, qblock = blockIdx.x;
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
   const int len = t1 - t0;
   if (len <= 0) return;
@@ -825,7 +827,7 @@ void attention_long_launch(const void* q, const void* k, const void* v, int layo
   auto kern = attention_long_kernel<T, NKT>;
   dim3 grid(NKT / 4, heads, batch);
   kern<<<grid, kAttnThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld, (const T*)attr_mask,
-                                             (T*)dst, seq_start, word_idx, seq_len, heads, scaler);
+                                             (T*)dst, seq_start, word_idx, batch, seq_len, heads, scaler);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -844,7 +846,7 @@ template <typename T>
 __global__ __launch_bounds__(kAttnThreads) void attention_generic_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
-    const int32_t* __restrict__ word_idx, int seq_len, int heads, int d, float scaler) {
+    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, int d, float scaler) {
   using C = Chunk16<T>;
   using V16 = typename C::vec;
   constexpr int kPerLane = kGenMaxSeq / kWave;             // keys per lane
@@ -852,7 +854,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_generic_kernel(
   __shared__ float prob[kAttnWaves][kGenMaxSeq];
   __shared__ float qrow[kAttnWaves][kGenMaxD];
 
-  const int b = blockIdx.z, head = blockIdx.y;
+  const int b = min(max(seq_start[batch + 1 + blockIdx.z], 0), batch - 1), head = blockIdx.y;
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
   const int len = t1 - t0;
   if (len <= 0) return;
@@ -949,8 +951,8 @@ void attention_generic_launch(const void* q, const void* k, const void* v, int l
                               int heads, int d, float scaler, hipStream_t stream) {
   dim3 grid((seq_len + kAttnWaves - 1) / kAttnWaves, heads, batch);
   attention_generic_kernel<T><<<grid, kAttnThreads, 0, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
-                                                                 (const T*)attr_mask, (T*)dst, seq_start, word_idx, seq_len,
-                                                                 heads, d, scaler);
+                                                                 (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch,
+                                                                 seq_len, heads, d, scaler);
 }
 
 template <typename T>

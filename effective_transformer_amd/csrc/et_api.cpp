@@ -140,7 +140,7 @@ LayerWs layer_ws(et_dtype dtype, int B, int S, int heads, int d) {
   w.ctx = off;   off += align_up(rows * H * e, 256);
   w.attn = off;  off += align_up(rows * H * e, 256);
   w.inter = off; off += align_up(rows * 4 * H * e, 256);
-  w.seq = off;   off += align_up(((size_t)B + 1) * sizeof(int32_t), 256);
+  w.seq = off;   off += align_up(et::seq_table_words(B) * sizeof(int32_t), 256);
   // fp16: k-contiguous copies of the six dense kernels (3 H^2 + H^2 + 4 H^2 + 4 H^2 elements) for the large-M GEMM
   w.wt = off;    off += dtype == ET_FP16 ? align_up(12 * H * H * e, 256) : 0;
   w.total = off;
@@ -250,7 +250,7 @@ size_t et_layer_workspace_bytes(et_dtype dtype, int batch_size, int seq_len, int
 
 size_t et_seq_workspace_bytes(int batch_size) {
   if (batch_size < 1) return 0;
-  return align_up(((size_t)batch_size + 1) * sizeof(int32_t), 256);
+  return align_up(et::seq_table_words(batch_size) * sizeof(int32_t), 256);
 }
 
 et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask, void* to_tensor,

@@ -1017,6 +1017,7 @@ void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, con
   a.seq = seq ? *seq : SeqStartJob{nullptr, nullptr, 0, 0, nullptr};
   if (seq) total += (seq->rows_bound + 1 + 255) / 256;
   layer_prologue_kernel<<<total, 256, 0, stream>>>(a);
+  if (seq) launch_seq_order(seq->seq_start, seq->batch, stream);
 }
 
 bool gemm_supported(DType t, int n, int k, int groups) {

@@ -250,6 +250,31 @@ __global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restric
   seq_start_for_row(batch_idx, T, blockIdx.x * 256 + threadIdx.x, batch, seq_start);
 }
 
+// order[0..batch) = the sequences sorted by length, longest first (buckets of 16 tokens; the order inside a bucket is
+// whatever the atomics give: it only decides which workgroup of the attention kernel starts first).  One workgroup.
+constexpr int kOrderBuckets = 65;             // lengths up to 1024
+__global__ __launch_bounds__(1024) void seq_order_kernel(const int32_t* __restrict__ seq_start, int batch,
+                                                         int32_t* __restrict__ order) {
+  __shared__ int hist[kOrderBuckets], base[kOrderBuckets];
+  for (int i = threadIdx.x; i < kOrderBuckets; i += 1024) hist[i] = 0;
+  __syncthreads();
+  auto bucket_of = [&](int b) {
+    const int len = seq_start[b + 1] - seq_start[b];
+    return kOrderBuckets - 1 - min(max(len, 0) >> 4, kOrderBuckets - 1);      // longest first
+  };
+  for (int b = threadIdx.x; b < batch; b += 1024) atomicAdd(&hist[bucket_of(b)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int i = 0; i < kOrderBuckets; ++i) {
+      base[i] = run;
+      run += hist[i];
+    }
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < batch; b += 1024) order[atomicAdd(&base[bucket_of(b)], 1)] = b;
+}
+
 // to[b,:] = row of the packed matrix that sits at position 0 of sequence b, zeros where sequence b has no token
 // there.  One wavefront per packed row (plus one past the end): the row that opens a sequence serves that sequence
 // and zeroes the token-less sequences in front of it, like seq_start_kernel walks the batch.
@@ -327,10 +352,15 @@ void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, c
                                                          n_pos, seq_len, row_bytes / 16);
 }
 
+void launch_seq_order(int32_t* seq_table, int batch, hipStream_t stream) {
+  seq_order_kernel<<<1, 1024, 0, stream>>>(seq_table, batch, seq_table + batch + 1);
+}
+
 void launch_seq_start(const int32_t* batch_idx, const int32_t* rows_dev, int rows_bound, int batch,
                       int32_t* seq_start, hipStream_t stream) {
   const int n = rows_bound + 1;
   seq_start_kernel<<<(n + 255) / 256, 256, 0, stream>>>(batch_idx, rows_dev, rows_bound, batch, seq_start);
+  launch_seq_order(seq_start, batch, stream);
 }
 
 }  // namespace et

@@ -40,9 +40,13 @@ void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, c
 // to[b,:] = packed row at position 0 of sequence b (zeros if there is none); indices ascending.
 void launch_first_token(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
                         const int32_t* rows_dev, int rows_bound, int batch, int row_bytes, hipStream_t stream);
-// seq_start[b] = first packed row of sequence b, b in [0,B]; seq_start[B] = T.
+// The sequence table of a batch, 2 B + 1 words: seq_start[b] = first packed row of sequence b, b in [0,B];
+// seq_start[B] = T; then the B sequence numbers in the order the attention kernels serve them (longest first).
+inline size_t seq_table_words(int batch) { return 2 * (size_t)batch + 1; }
 void launch_seq_start(const int32_t* batch_idx, const int32_t* rows_dev, int rows_bound, int batch,
                       int32_t* seq_start, hipStream_t stream);
+// second half of the table from its first half (for tables whose first half another kernel wrote)
+void launch_seq_order(int32_t* seq_table, int batch, hipStream_t stream);
 
 // ---- row_kernels.hip ---------------------------------------------------------------------
 bool bias_gelu_supported(DType t, int n);

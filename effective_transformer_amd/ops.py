@@ -285,12 +285,16 @@ def effective_transformer(from_tensor: torch.Tensor, to_tensor: torch.Tensor, at
 
 def sequence_starts(valid_word_num: torch.Tensor, batch_idx: torch.Tensor, batch_size: int, seq_len: int,
                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """int32[batch_size + 1]: first packed row of every sequence (entry batch_size = valid-token count), the table
-    the attention kernel walks; one per batch serves all layers."""
+    """The sequence table of a batch, int32[2 * batch_size + 1]: first packed row of every sequence (entry batch_size
+    = valid-token count), then the sequence numbers in the order the attention kernel serves them (longest first); one
+    per batch serves all layers."""
     lib = _lib.load()
     _require_cuda(valid_word_num, batch_idx)
+    words = lib.et_seq_workspace_bytes(batch_size) // 4
     if out is None:
-        out = torch.empty(batch_size + 1, dtype=torch.int32, device=batch_idx.device)
+        out = torch.empty(words, dtype=torch.int32, device=batch_idx.device)
+    elif out.numel() < 2 * batch_size + 1:
+        raise ValueError("the sequence table holds 2 * batch_size + 1 int32")
     h = handle(batch_idx.device)
     _lib.check(lib.et_sequence_starts(h, _p(batch_idx), _p(valid_word_num), batch_size, seq_len, _p(out), _stream()), h)
     return out
@@ -389,7 +393,8 @@ class EffectiveTransformerEncoder:
         key = tuple(x.shape)
         bufs = self._bufs.get(key)
         if bufs is None:
-            bufs = (torch.empty_like(x), torch.empty_like(x), torch.empty(B + 1, dtype=torch.int32, device=x.device))
+            bufs = (torch.empty_like(x), torch.empty_like(x),
+                    torch.empty(2 * B + 1, dtype=torch.int32, device=x.device))
             self._bufs[key] = bufs
         starts = sequence_starts(vwn, bidx, B, S, out=bufs[2])       # one table for all layers of the batch
         for l, w in enumerate(self.layers):

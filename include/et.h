@@ -81,7 +81,8 @@ typedef struct et_layer_weights {
  * bytes but indexes it in elements, tf_op/bert_transformer_op.cu.cc:75-96). */
 size_t et_input_workspace_bytes(int batch_size, int seq_len);
 size_t et_layer_workspace_bytes(et_dtype dtype, int batch_size, int seq_len, int head_num, int size_per_head);
-/* scratch for the per-sequence start table some kernel-level entry points build */
+/* size of the sequence table of a batch (et_sequence_starts; also the scratch of the kernel-level entry points that
+ * build one): 2 * batch_size + 1 int32, rounded up to 256 bytes */
 size_t et_seq_workspace_bytes(int batch_size);
 
 /* ---- the three ops ------------------------------------------------------------------ */
@@ -131,7 +132,7 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
  *   *_t: the dense kernel handed over [out,in] (k-contiguous), i.e. et_transpose_weight of the [in,out] tensor, fp16
  *        only.  Used where et_layer would run its large-M GEMM (it then skips its per-call transposition; Q, K and V
  *        go together); ignored for batches that run the small-M kernels, which read the [in,out] tensors.
- *   seq_start: int32[batch_size + 1] from et_sequence_starts for THIS batch (first packed row of every sequence);
+ *   seq_start: the sequence table et_sequence_starts wrote for THIS batch (et_seq_workspace_bytes(batch_size) bytes);
  *        the same table serves every layer of the batch. */
 typedef struct et_layer_prepared {
   const void* attr_kernel_Q_t;       /* [H,H]  */
@@ -140,12 +141,14 @@ typedef struct et_layer_prepared {
   const void* attr_output_kernel_t;  /* [H,H]  */
   const void* inter_kernel_t;        /* [4H,H] */
   const void* output_kernel_t;       /* [H,4H] */
-  const int32_t* seq_start;          /* [B+1]  */
+  const int32_t* seq_start;          /* [2B+1] */
 } et_layer_prepared;
 
-/* seq_start[b] = first packed row of sequence b for b in [0,B), seq_start[B] = T: the table the attention kernel
- * walks, from the index arrays et_input produced.  No counterpart in the reference (its attention works on padded
- * buffers). */
+/* The sequence table of a batch, from the index arrays et_input produced: seq_start[b] = first packed row of sequence
+ * b for b in [0,B), seq_start[B] = T, followed by the B sequence numbers in the order the attention kernels serve them
+ * (by length, longest first: workgroups of similar duration run side by side and the long ones start first).
+ * seq_start must hold et_seq_workspace_bytes(batch_size) bytes (2 B + 1 int32).  No counterpart in the reference (its
+ * attention works on padded buffers). */
 et_status et_sequence_starts(et_handle h, const int32_t* batch_idx, const int32_t* valid_word_num_dev, int batch_size,
                              int seq_len, int32_t* seq_start, void* stream);
 
@@ -271,9 +274,10 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
                        const int32_t* batch_idx, const int32_t* word_idx,
                        void* workspace, size_t workspace_bytes, void* stream);
 
-/* et_attention with the sequence start table of et_sequence_starts handed in (seq_start, int32[B+1]; one table serves
+/* et_attention with the sequence start table of et_sequence_starts handed in (seq_start; one table serves
  * every layer of a batch, as in et_layer_with_prepared), so that the call is the attention kernel alone.  With
- * seq_start NULL the table is built into seq_start_scratch (int32[B+1]) first, which is what et_attention does.  No
+ * seq_start NULL the table is built into seq_start_scratch (et_seq_workspace_bytes(B) bytes) first, which is what
+ * et_attention does.  No
  * counterpart in the reference, whose attention works on padded buffers. */
 et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v,
                                    int qkv_layout, int packed_ld, const void* attr_mask, void* dst,

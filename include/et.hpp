@@ -111,7 +111,8 @@ class Encoder {
     const size_t e = dtype_ == ET_FP32 ? 4 : 2;
     const size_t H = (size_t)heads_ * d_, rows = (size_t)batch * seq_len;
     char* act = (char*)act_.reserve(3 * rows * H * e);                 // packed input + two layer outputs
-    int32_t* idx = (int32_t*)idx_.reserve((2 * rows + 1 + (size_t)batch + 1) * sizeof(int32_t));
+    // batch_idx, word_idx, the count, then the sequence table (2 B + 1 words)
+    int32_t* idx = (int32_t*)idx_.reserve((2 * rows + 1) * sizeof(int32_t) + et_seq_workspace_bytes(batch));
     int32_t *batch_idx = idx, *word_idx = idx + rows, *count = idx + 2 * rows, *starts = idx + 2 * rows + 1;
     const size_t in_ws = et_input_workspace_bytes(batch, seq_len);
     const size_t layer_ws = et_layer_workspace_bytes(dtype_, batch, seq_len, heads_, d_);
