@@ -559,15 +559,30 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
   const int xcd = blockIdx.x % kXcds;
   const int G = gridDim.x;                                        // multiple of 8
 
-  auto tile_id = [&](int idx) { return xcd * per_xcd + idx / kXcds; };
-  auto valid = [&](int idx) { return idx / kXcds < per_xcd && tile_id(idx) < total; };
+  // This XCD's band holds n_loc tiles for wgs workgroups: `full` of them fill whole rounds.  When the rest would keep at
+  // most half of the workgroups busy for a last round, each of those tiles is shared by two workgroups, one per
+  // 128-column half: the waves of the other half only keep the operand stream going, a SIMD then has one MFMA wave
+  // instead of two, and the last round takes about half a tile time.  Every element is still accumulated by one wave in
+  // the same k order, so the bits do not depend on the split.
+  const int wgs = G / kXcds, local = blockIdx.x / kXcds;
+  const int n_loc = max(0, min(per_xcd, total - xcd * per_xcd));
+  const int full = (n_loc / wgs) * wgs, rem = n_loc - full;
+  const bool split = rem > 0 && 2 * rem <= wgs;
+  // slot s (= local + round * wgs) of the band -> tile and half (-1: the whole tile)
+  auto valid = [&](int s) { return s < full || (split ? s - full < 2 * rem : s < n_loc); };
 
   struct Src {
     __amdgpu_buffer_rsrc_t a, b;
-    int m0, n0, grp;
+    int m0, n0, grp, half;
   };
-  auto locate = [&](int tile) {
+  auto locate = [&](int s) {
     Src t;
+    t.half = -1;
+    int tile = xcd * per_xcd + s;
+    if (s >= full && split) {
+      t.half = (s - full) & 1;
+      tile = xcd * per_xcd + full + ((s - full) >> 1);
+    }
     if (args.reverse_walk) tile = total - 1 - tile;
     const int tm = tile / tiles_n_all;
     const int tn_all = tile - tm * tiles_n_all;
@@ -609,23 +624,22 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
   const int b_rd[2] = {kQAPair + (wn * 64 + l16) * 128 + ((g ^ sw) * 16),
                        kQAPair + (wn * 64 + l16) * 128 + (((4 + g) ^ sw) * 16)};
 
-  int idx = blockIdx.x;
+  int idx = local;
   if (!valid(idx)) return;
   {
     // The workgroups of an XCD run their tiles in lockstep, so all of them stream operands and store C at the same
     // moments.  Those that walk one tile less than the others have a tile time to spare: they start late, spread over
     // about a quarter of a tile time (960 cycles per pair of k-steps), which takes their traffic out of step with the
     // rest at no cost to the last round (measured: -1.3 % on the encoder step, nothing gained beyond that spread).
-    const int wgs = G / kXcds, local = blockIdx.x / kXcds;
-    const int n_loc = min(per_xcd, total - xcd * per_xcd);
     const int max_tiles = (n_loc + wgs - 1) / wgs;
-    const int first_short = n_loc - (max_tiles - 1) * wgs;      // first workgroup of this XCD with max_tiles - 1 tiles
+    // first workgroup of this XCD with max_tiles - 1 tiles
+    const int first_short = split ? 2 * rem : n_loc - (max_tiles - 1) * wgs;
     if (local >= first_short && first_short < wgs) {
       const int units = (np * 15 + 90) * (local - first_short + 1) / (wgs - first_short + 1);   // of 64 cycles
       for (int u = 0; u < units; u += 16) __builtin_amdgcn_s_sleep(16);
     }
   }
-  Src cur = locate(tile_id(idx)), nxt = cur;
+  Src cur = locate(idx), nxt = cur;
 
   float4v acc[8][4];
   half8 a[2][8], b[2][4];
@@ -674,27 +688,44 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
 
   bool first_tile = true;
   while (true) {
-    const int nidx = idx + G;
+    const int nidx = idx + wgs;
     const bool has_next = valid(nidx);
-    if (has_next) nxt = locate(tile_id(nidx));   // otherwise the stream re-loads this tile; the data is never used
-    for (int p = 0; p < np; ++p) {
-      const int s = pairs_done & 1;
-      if (p == 0) step(Even{}, std::true_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
-      else step(Even{}, std::false_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
-      // this wave's share of the next pair has landed (right after a tile boundary that was confirmed before the C
-      // stores went out) and its last reads of slot s, which feed the odd step, are complete
-      if (first_tile || p >= 1) wait_vmcnt<0>();
-      wait_lgkmcnt0();
-      barrier_only();
-      // pair p+2 of this tile, or the matching pair of the next one, replaces slot s
-      const bool in_tile = p + 2 < np;
-      const __amdgpu_buffer_rsrc_t da = in_tile ? cur.a : nxt.a;
-      const __amdgpu_buffer_rsrc_t db = in_tile ? cur.b : nxt.b;
-      step(Odd{}, std::false_type{}, std::true_type{}, s ^ 1, s, in_tile ? p + 2 : p + 2 - np, da, db);
-      ++pairs_done;
+    if (has_next) nxt = locate(nidx);            // otherwise the stream re-loads this tile; the data is never used
+    // a shared tile: this wave computes only when its columns lie in the workgroup's half
+    const bool computes = cur.half < 0 || (wn >> 1) == cur.half;
+    if (computes) {
+      for (int p = 0; p < np; ++p) {
+        const int s = pairs_done & 1;
+        if (p == 0) step(Even{}, std::true_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
+        else step(Even{}, std::false_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
+        // this wave's share of the next pair has landed (right after a tile boundary that was confirmed before the C
+        // stores went out) and its last reads of slot s, which feed the odd step, are complete
+        if (first_tile || p >= 1) wait_vmcnt<0>();
+        wait_lgkmcnt0();
+        barrier_only();
+        // pair p+2 of this tile, or the matching pair of the next one, replaces slot s
+        const bool in_tile = p + 2 < np;
+        const __amdgpu_buffer_rsrc_t da = in_tile ? cur.a : nxt.a;
+        const __amdgpu_buffer_rsrc_t db = in_tile ? cur.b : nxt.b;
+        step(Odd{}, std::false_type{}, std::true_type{}, s ^ 1, s, in_tile ? p + 2 : p + 2 - np, da, db);
+        ++pairs_done;
+      }
+    } else {
+      // the other half's waves: same barriers, same share of the DMA, no operand reads and no MFMAs
+      for (int p = 0; p < np; ++p) {
+        const int s = pairs_done & 1;
+        if (first_tile || p >= 1) wait_vmcnt<0>();
+        barrier_only();
+        const bool in_tile = p + 2 < np;
+        const __amdgpu_buffer_rsrc_t da = in_tile ? cur.a : nxt.a;
+        const __amdgpu_buffer_rsrc_t db = in_tile ? cur.b : nxt.b;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) issue1(s, in_tile ? p + 2 : p + 2 - np, da, db, q);
+        ++pairs_done;
+      }
     }
     wait_vmcnt<0>();
-    {
+    if (computes) {
       // C leaves through a descriptor that covers the tile's valid rows only: rows beyond them are dropped by the
       // bounds check, and the only per-store address arithmetic is one add on the running byte offset
       const int col = cur.n0 + wn * 64 + l16 * 4;

@@ -364,7 +364,10 @@ def test_gemm(k, dtype, m, n, k_):
 
 # The k-contiguous-B kernel only runs from 128 tiles of 256x256 on: shapes are sized for that, the
 # oracle product is taken on the CPU in float64 for a sample of rows.
-@pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072)])
+# The last two shapes leave a last round that keeps at most half of the workgroups busy: those tiles are shared by two
+# workgroups, one per 128-column half (one of them with a ragged last column tile).
+@pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072),
+                                    (23301, 768, 768), (14000, 1032, 128)])
 def test_gemm_bt(k, m, n, k_):
     print("gemm_bt", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_)
