@@ -516,11 +516,11 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
   auto kern = attention_kernel<T, NKT, CPT, PF>;
   allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Sm::kBytes);
   // A workgroup serves several heads of one sequence: mask rows, positions and zero fill are shared by them, and the
-  // chain of dependent loads a workgroup starts with (sequence start, positions, rows) is paid once.  Up to 4 heads
-  // (8 for the 128-key kernel, whose start is the longest), in equal groups, as long as about two workgroups per CU
+  // chain of dependent loads a workgroup starts with (sequence start, positions, rows) is paid once.  Up to 6 heads
+  // (4 in fp32; 8 for the 128-key kernel, whose start is the longest), in equal groups, as long as about two workgroups per CU
   // remain: measured best on batches of 100 x 32, 1000 x 64 and 256 x 128 tokens.
   int hpw = 1;
-  for (int h = NKT >= 8 ? 8 : 4; h > 1; --h)
+  for (int h = NKT >= 8 ? 8 : (sizeof(T) == 2 ? 6 : 4); h > 1; --h)
     if (heads % h == 0 && (long)batch * (heads / h) >= 512) {
       hpw = h;
       break;
