@@ -109,9 +109,10 @@ def _time_kernel(fn, iters, warm=3):
     return s.elapsed_time(e) / iters          # ms per launch
 
 
-def per_kernel(wl, T, mask_np, iters=20):
+def per_kernel(wl, T, mask_np, iters=20, vendor_gemm=False):
     """Times every kernel of the path in isolation at the workload's real shapes and prices it
-    against its roofline with ALGORITHMIC bytes / flops."""
+    against its roofline with ALGORITHMIC bytes / flops.  vendor_gemm: also time the vendor library's GEMM
+    (torch.matmul) on the same operands in the same kind of launch loop, as a calibration point."""
     import numpy as np
     import torch
     from effective_transformer_amd import kernel_ops as k, ops
@@ -196,6 +197,7 @@ def per_kernel(wl, T, mask_np, iters=20):
         Cm = torch.empty(T, n, device="cuda", dtype=dt)
         kw = {"bias": bF, "gelu": True} if name == "gemm_ffn_up" else {}
         fn = lambda: k.gemm(A, Bm, out=Cm, **kw)
+        plain = lambda: k.gemm(A, Bm, out=Cm)
         if dt == torch.float16:
             # the encoder object hands k-contiguous copies of its (constant) weights to the layer op, which runs them
             # on the large-M kernel once the batch fills the chip
@@ -203,12 +205,26 @@ def per_kernel(wl, T, mask_np, iters=20):
             try:
                 k.gemm_bt(A, Bt, out=Cm, **kw)
                 fn = lambda: k.gemm_bt(A, Bt, out=Cm, **kw)
+                plain = lambda: k.gemm_bt(A, Bt, out=Cm)
             except Exception:
                 pass
         ms = _time_kernel(fn, iters)
         add(name, ms, "mfma", 2.0 * T * n * kk)
         if kw:
             res[name]["epilogue"] = "bias+gelu"
+        if vendor_gemm:
+            # calibration only, never on the path: the plain product (no bias, no GELU) by the vendor library, with the
+            # weights in TF's [k][n] order and in the k-contiguous [n][k] order
+            Bnk = Bm.t().contiguous()
+            try:
+                v_kn = _time_kernel(lambda: torch.matmul(A, Bm, out=Cm), iters)
+                v_nk = _time_kernel(lambda: torch.matmul(A, Bnk.t(), out=Cm), iters)
+                res[name]["vendor"] = {"library": "torch.matmul (hipBLASLt / rocBLAS), plain product",
+                                       "ms_weights_kn": round(v_kn, 5), "ms_weights_nk": round(v_nk, 5)}
+                if kw:      # the own kernel without the epilogue, for a like-for-like number
+                    res[name]["ms_plain_product"] = round(_time_kernel(plain, iters), 5)
+            except Exception as ex:       # a library failure must not take the benchmark line down
+                res[name]["vendor"] = {"error": str(ex)[:200]}
     if dt == torch.float16:
         Wall = rnd(H, 7 * H)                          # Q, K, V and FFN-up kernels
         Wt = torch.empty(7 * H, H, device="cuda", dtype=dt)
@@ -338,6 +354,8 @@ def main():
     ap.add_argument("--cpu-seqs", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--calibrate-gemm", action="store_true",
+                    help="also time the vendor library's GEMM (torch.matmul) on the four projection shapes")
     ap.add_argument("--fold-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no benchmark: fold two rocprofv3 --pmc counter files into profiles/hbm_traffic.json")
     ap.add_argument("--commit", default="unknown", help="with --fold-traffic: the commit the counters were measured on")
@@ -400,7 +418,7 @@ def main():
         torch.cuda.synchronize()
         graph_ms = s.elapsed_time(e) / a.steps
         del g
-    kernels = {} if a.no_kernels else per_kernel(wl, T, w["mask"])
+    kernels = {} if a.no_kernels else per_kernel(wl, T, w["mask"], vendor_gemm=a.calibrate_gemm)
     roof = None
     layer_sum = None
     if kernels:

@@ -772,7 +772,7 @@ et_status gemm_bt_impl(et_handle h, et_dtype dtype, const void* A, const void* B
   if ((uint64_t)m * k * 2 > 0xffffffffull) return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
   if (!et::gemm_takes_transposed_b(et::DType::F16, m, n, n, k, 1))
     return fail(h, ET_UNSUPPORTED,
-                std::string(what) + " needs k % 64 == 0, n % 8 == 0 and at least 128 tiles of 256x256");
+                std::string(what) + " needs k % 64 == 0 and n % 8 == 0");
   et::GemmGroups g;
   g.groups = 1;
   g.A[0] = A; g.B[0] = Bt; g.bias[0] = bias;

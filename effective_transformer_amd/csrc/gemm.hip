@@ -771,6 +771,179 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
 }
 
 // ------------------------------------------------------------------------------------------
+// fp16, problems below the persistent regime, B k-contiguous ([n][k]): one (32 MI) x (32 NJ) tile per workgroup,
+// 4 wavefronts (2 x 2), LDS slots of two k-steps like the persistent kernel above.
+//
+// With the weights in TF's [k][n] order a small tile reads its B operands with 8-byte LDS reads (half the rate of
+// 16-byte ones) and transposes them in registers, and its A rows arrive in 64-byte pieces; a 64 x 128 tile then spends
+// about three times as long on LDS traffic, transposes and DMA issue as on its 8 MFMAs per k-step, with one wavefront
+// per SIMD and nothing to overlap them with.  Here both operands are rows of 64 k = 128 bytes (full cache lines for the
+// DMA), every operand read is one 16-byte read per 16 x 32 block, and there are no transposes.  The ring holds ST slots;
+// the schedule is the persistent kernel's: even k-step, barrier, odd k-step with this wave's DMA for the pair ST ahead.
+// ------------------------------------------------------------------------------------------
+template <int MI, int NJ, int ST>
+struct BtTile {
+  static constexpr int BM = 32 * MI, BN = 32 * NJ;
+  static constexpr int A_BYTES = BM * 128;
+  static constexpr int SLOT_BYTES = (BM + BN) * 128;
+  static constexpr int SMEM_BYTES = ST * SLOT_BYTES;
+  static constexpr int DMA = MI + NJ;                         // instructions per wavefront and pair: MI for A, NJ for B^T
+};
+
+template <int MI, int NJ, int ST>
+__global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f16_bt_kernel(GemmArgs args) {
+#if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
+  using Tile = BtTile<MI, NJ, ST>;
+  static_assert(Tile::DMA * (ST - 1) < 64, "the DMA instructions in flight must fit the 6-bit vmcnt");
+  using HalfN = typename std::conditional<NJ == 8, half8, typename std::conditional<NJ == 4, half4, half2v>::type>::type;
+  constexpr int BM = Tile::BM, BN = Tile::BN, WC = 16 * NJ;       // WC: columns of a wave tile
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
+  const int tiles_n_all = args.tiles_n * args.groups;
+  const int tile = remap_valid_tile(blockIdx.x, ((rows + BM - 1) / BM) * tiles_n_all);
+  if (tile < 0) return;
+  const int tm = tile / tiles_n_all;
+  const int tn_all = tile - tm * tiles_n_all;
+  const int grp = tn_all / args.tiles_n;
+  const int m0 = tm * BM;
+  const int n0 = (tn_all - grp * args.tiles_n) * BN;
+  const int N = args.n, K = args.k;
+  const int np = K / 64;                                          // pairs of k-steps
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // scalar: LDS targets of the DMA are SALU values
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, g = lane >> 4;
+
+  // descriptors start at the tile and end with the matrix: rows at or beyond the valid-token count and columns at or
+  // beyond n read as zero, and lane offsets do not grow with the matrices
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16*>((const _Float16*)args.A[grp] + (size_t)m0 * K), 0, min(rows - m0, BM) * K * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16*>((const _Float16*)args.B[grp] + (size_t)n0 * K), 0, min(N - n0, BN) * K * 2, 0x00020000);
+
+  // DMA: one instruction fills 1 KB of LDS = 8 rows x 128 bytes; the lane picks the 16-byte chunk that belongs at its
+  // (XOR-swizzled) position.  LDS row j*16+l of a wave's column group holds column NJ*l+j of the group, so that the
+  // operand reads of B^T look like A's and a lane owns NJ consecutive columns of C.
+  uint32_t voff_a[MI], voff_b[NJ];
+#pragma unroll
+  for (int j = 0; j < MI; ++j) {
+    const int row = wave * (8 * MI) + j * 8 + (lane >> 3);
+    voff_a[j] = ((uint32_t)row * (uint32_t)K + (uint32_t)((lane & 7) ^ pair_swizzle(row)) * 8u) * 2u;
+  }
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int row = wave * (8 * NJ) + j * 8 + (lane >> 3);
+    const int col = (row / WC) * WC + (row & 15) * NJ + ((row % WC) >> 4);
+    voff_b[j] = ((uint32_t)col * (uint32_t)K + (uint32_t)((lane & 7) ^ pair_swizzle(row)) * 8u) * 2u;
+  }
+  // instruction q (0..MI-1: A, MI..: B^T) of this wave's share of pair `pr` into slot `slot`; pairs past the end
+  // re-load the last one (never used; keeps the DMA count uniform)
+  auto issue1 = [&](int slot, int pr, int q) {
+    unsigned char* st = smem + slot * Tile::SLOT_BYTES;
+    const int koff = min(pr, np - 1) * 128;
+    if (q < MI)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, ET_LDS_PTR(st + (wave * MI + q) * 1024), 16, voff_a[q], koff, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, ET_LDS_PTR(st + Tile::A_BYTES + (wave * NJ + q - MI) * 1024), 16,
+                                               voff_b[q - MI], koff, 0, 0);
+  };
+
+  // operand reads: row (wm*16*MI + i*16 + l16) resp. (wn*WC + j*16 + l16), chunk (4*half + g), swizzled
+  const int sw = pair_swizzle(l16);
+  const int a_rd[2] = {(wm * 16 * MI + l16) * 128 + ((g ^ sw) * 16), (wm * 16 * MI + l16) * 128 + (((4 + g) ^ sw) * 16)};
+  const int b_rd[2] = {Tile::A_BYTES + (wn * WC + l16) * 128 + ((g ^ sw) * 16),
+                       Tile::A_BYTES + (wn * WC + l16) * 128 + (((4 + g) ^ sw) * 16)};
+
+  float4v acc[MI][NJ];
+  half8 a[2][MI], b[2][NJ];
+
+  // One k-step: MFMAs on operand set P; half 1-P of slot `rs` is read into the other set (B^T blocks first: the first
+  // MFMAs of the next step need all of them); with DMA set, this wave's instructions for pair `dpr` go into slot `ds`.
+  auto step = [&](auto Pc, auto FIRSTc, auto DMAc, int rs, int ds, int dpr) {
+    constexpr int P = decltype(Pc)::value;
+    constexpr bool FIRST = decltype(FIRSTc)::value;
+    constexpr bool DMA = decltype(DMAc)::value;
+    constexpr int rh = 1 - P;                    // the even step reads half 1 of its own pair, the odd step half 0 of the next
+    constexpr int kRpg = (MI + NJ + MI - 1) / MI, kDpg = (Tile::DMA + MI - 1) / MI;
+    const unsigned char* ns = smem + rs * Tile::SLOT_BYTES;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int r = i * kRpg; r < (i + 1) * kRpg && r < MI + NJ; ++r) {
+        if (r < NJ) b[1 - P][r] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + r * 2048);
+        else a[1 - P][r - NJ] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (r - NJ) * 2048);
+      }
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[P][i], b[P][j],
+                                                           FIRST ? float4v{0.f, 0.f, 0.f, 0.f} : acc[i][j], 0, 0, 0);
+      if (DMA) {
+#pragma unroll
+        for (int q = i * kDpg; q < (i + 1) * kDpg && q < Tile::DMA; ++q) issue1(ds, dpr, q);
+      }
+      __builtin_amdgcn_sched_barrier(0);         // keeps the reads and the DMA where they are between the MFMA groups
+    }
+  };
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+
+#pragma unroll
+  for (int s = 0; s < ST; ++s)
+#pragma unroll
+    for (int q = 0; q < Tile::DMA; ++q) issue1(s, s, q);
+  wait_vmcnt<Tile::DMA * (ST - 1)>();
+  barrier_only();
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) b[0][j] = *reinterpret_cast<const half8*>(smem + b_rd[0] + j * 2048);
+#pragma unroll
+  for (int i = 0; i < MI; ++i) a[0][i] = *reinterpret_cast<const half8*>(smem + a_rd[0] + i * 2048);
+
+  int s = 0;                                     // slot of pair p
+  for (int p = 0; p < np; ++p) {
+    if (p == 0) step(Even{}, std::true_type{}, std::false_type{}, s, 0, 0);
+    else step(Even{}, std::false_type{}, std::false_type{}, s, 0, 0);
+    wait_vmcnt<Tile::DMA * (ST - 2)>();          // this wave's share of pair p+1 has landed; the ST - 2 behind it may fly
+    wait_lgkmcnt0();                             // its last reads of slot s, which feed the odd step, are complete
+    barrier_only();
+    const int s1 = s + 1 == ST ? 0 : s + 1;
+    step(Odd{}, std::false_type{}, std::true_type{}, s1, s, p + ST);      // pair p+ST replaces slot s
+    s = s1;
+  }
+  wait_vmcnt<0>();                               // no DMA may still target this workgroup's LDS when it ends
+
+  // epilogue: lane owns rows g*4+r of every 16-row block and NJ consecutive columns
+  const int col = n0 + wn * WC + l16 * NJ;
+  if (col < N) {
+    _Float16* C = (_Float16*)args.C + (size_t)grp * N + col;
+    // bias added in half on the rounded product, as the reference's next kernel does; without a bias the addend is
+    // -0, which leaves every value (and the sign of a zero) as it is
+    HalfN biasv;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) biasv[j] = (_Float16)-0.0f;
+    if (args.bias[grp] != nullptr) biasv = *reinterpret_cast<const HalfN*>((const _Float16*)args.bias[grp] + col);
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = m0 + wm * 16 * MI + i * 16 + g * 4 + r;
+        if (row < rows) {
+          HalfN o;
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) o[j] = f2h(acc[i][j][r]);
+          o = args.gelu ? bias_gelu_half<HalfN, NJ>(o, biasv) : o + biasv;
+          __builtin_nontemporal_store(o, reinterpret_cast<HalfN*>(C + (size_t)row * args.ldc));
+        }
+      }
+  }
+#else
+  (void)args;
+#endif
+}
+
+// ------------------------------------------------------------------------------------------
 // fp32: 128x128x16 tile, 4 wavefronts (2x2) of 64x64, v_mfma_f32_32x32x2_f32
 // ------------------------------------------------------------------------------------------
 constexpr int kFThreads = 256;
@@ -935,6 +1108,18 @@ void launch_f16(GemmArgs a, hipStream_t stream) {
   kern<<<a.per_xcd * kXcds, kHThreads, Tile::SMEM_BYTES, stream>>>(a);
 }
 
+template <int MI, int NJ, int ST>
+void launch_f16_bt(GemmArgs a, hipStream_t stream) {
+  using Tile = BtTile<MI, NJ, ST>;
+  auto kern = gemm_f16_bt_kernel<MI, NJ, ST>;
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Tile::SMEM_BYTES);
+  a.tiles_m = (a.m_bound + Tile::BM - 1) / Tile::BM;
+  a.tiles_n = (a.n + Tile::BN - 1) / Tile::BN;
+  const int total = a.tiles_m * a.tiles_n * a.groups;
+  a.per_xcd = (total + kXcds - 1) / kXcds;
+  kern<<<a.per_xcd * kXcds, kHThreads, Tile::SMEM_BYTES, stream>>>(a);
+}
+
 int device_cu_count() {
   constexpr int kMaxDevices = 64;
   static std::atomic<int> cus[kMaxDevices] = {};      // handles on several GPUs may launch from different threads
@@ -1025,14 +1210,16 @@ __global__ __launch_bounds__(256) void layer_prologue_kernel(TransposeArgs args)
 }  // namespace
 
 bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
-  return t == DType::F16 && gemm_supported(t, n, k, groups) && k % 64 == 0 && use_persistent(m_bound, ldc, n, k, groups);
+  (void)m_bound; (void)ldc;
+  return t == DType::F16 && gemm_supported(t, n, k, groups) && k % 64 == 0 && (uint64_t)k * 256u * 2u < 0x80000000ull;
 }
 
 // Inside the layer the transposed copy pays off for the wide projections (QKV, FFN up: many column tiles re-read a
 // short k extent).  With k >= n the activations stream through L2 once per few tiles and the [k][n] kernel, whose B rows
 // are 512 contiguous bytes, is as fast inside the layer as the k-contiguous one is on its own, so the copy is skipped.
 bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
-  return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && (long)n * groups >= 2L * k;
+  return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && use_persistent(m_bound, ldc, n, k, groups) &&
+         (long)n * groups >= 2L * k;
 }
 
 void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, const SeqStartJob* seq) {
@@ -1077,6 +1264,27 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   if (t == DType::F16) {
     if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
       launch_f16_persistent(a, stream, g.b_transposed);
+    } else if (g.b_transposed) {
+      // Below the persistent regime a workgroup's k loop runs at the rate its CU's load path delivers the operand rows
+      // (the smaller the tile, the more bytes per MFMA), so the largest tile that still gives about 0.55 workgroups
+      // per CU is taken; the ring is deeper (5 or 6 slots) when every workgroup has a CU to itself, and small enough
+      // for two workgroups per CU otherwise (timed for n = 768 .. 3072, k = 768 and 3072, 250 .. 10000 rows, with the
+      // weights of twelve layers taking turns).
+      const int cus = device_cu_count();
+      auto wgs = [&](int bm, int bn) { return (long)((m_bound + bm - 1) / bm) * ((n + bn - 1) / bn) * g.groups; };
+      const long enough = (long)cus * 55 / 100;
+      if (wgs(128, 128) >= enough) {
+        if (wgs(128, 128) <= cus) launch_f16_bt<4, 4, 5>(a, stream);
+        else launch_f16_bt<4, 4, 2>(a, stream);
+      } else if (wgs(64, 128) >= enough) {
+        if (wgs(64, 128) <= cus) launch_f16_bt<2, 4, 6>(a, stream);
+        else launch_f16_bt<2, 4, 3>(a, stream);
+      } else if (wgs(64, 64) >= enough) {
+        if (wgs(64, 64) <= cus) launch_f16_bt<2, 2, 6>(a, stream);
+        else launch_f16_bt<2, 2, 3>(a, stream);
+      } else {
+        launch_f16_bt<1, 2, 6>(a, stream);
+      }
     } else {
       // Below a round of the chip the time of a launch is the k loop of one tile.  With fewer 64 x 256 tiles than CUs
       // that loop runs at the rate one CU's DMA fills its LDS: the 64 x 128 tile halves the B bytes per workgroup and

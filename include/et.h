@@ -303,17 +303,17 @@ et_status et_gemm_bias_gelu(et_handle h, et_dtype dtype, const void* A, const vo
 et_status et_transpose_weight(et_handle h, et_dtype dtype, const void* src, void* dst, int k, int n, void* stream);
 
 /* et_gemm with the second operand k-contiguous: C[m,n] = A[m,k] . Bt[n,k]^T (+ bias), fp16 only.  This is the kernel
- * et_layer runs once a batch has enough tokens to fill the chip (same cublasGemmEx call sites as et_gemm);
- * ET_UNSUPPORTED for k % 64 != 0 and for shapes with fewer than 128 tiles of 256x256, which go through et_gemm's
- * kernels. */
+ * et_layer runs where it has such a copy of a weight (same cublasGemmEx call sites as et_gemm): a persistent kernel
+ * from 128 tiles of 256x256 on, one tile of 32x64 .. 128x128 per workgroup below that.  Same bits as et_gemm on the
+ * same operands.  ET_UNSUPPORTED for k % 64 != 0 or n % 8 != 0. */
 et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
                      int m, int n, int k, const int32_t* m_dev, void* stream);
 
 /* C[m,n] = gelu(A[m,k] . Bt[n,k]^T + bias[n]): et_gemm_bt with et_add_bias_act applied to each tile on its way out,
  * same arithmetic and rounding points as the two calls in a row (reference: the cublasGemmEx call and the
  * add_bias_act launch that follows it, tf_op/bert_transformer_op.cu.cc:215-227, cuda/cuda_kernels.cu:29-51, 88-150).
- * This is what et_layer runs for the first FFN projection of a large batch.  fp16 only, bias required; shapes as
- * for et_gemm_bt. */
+ * This is what et_layer runs for the first FFN projection where it has a k-contiguous copy of the weight.  fp16 only,
+ * bias required; shapes as for et_gemm_bt. */
 et_status et_gemm_bt_bias_gelu(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
                                int m, int n, int k, const int32_t* m_dev, void* stream);
 

@@ -362,12 +362,15 @@ def test_gemm(k, dtype, m, n, k_):
         assert np.array_equal(got2[:m - 5], got[:m - 5]) and np.all(got2[m - 5:] == 0)
 
 
-# The k-contiguous-B kernel only runs from 128 tiles of 256x256 on: shapes are sized for that, the
-# oracle product is taken on the CPU in float64 for a sample of rows.
-# The last two shapes leave a last round that keeps at most half of the workgroups busy: those tiles are shared by two
-# workgroups, one per 128-column half (one of them with a ragged last column tile).
+# The k-contiguous-B kernels: the persistent 256x256 one from 128 such tiles on (first six shapes; the last two of
+# those leave a last round that keeps at most half of the workgroups busy, so those tiles are shared by two
+# workgroups, one per 128-column half, one of them with a ragged last column tile), below that one tile per workgroup
+# of 128x128 (one or two workgroups per CU), 64x128, 64x64 or 32x64, with ragged last tiles in both directions and a
+# single pair of k-steps.  The oracle product is taken on the CPU in float64 for a sample of rows.
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072),
-                                    (23301, 768, 768), (14000, 1032, 128)])
+                                    (23301, 768, 768), (14000, 1032, 128),
+                                    (6000, 776, 768), (4000, 768, 3072), (3000, 1032, 128), (2000, 768, 768),
+                                    (1001, 776, 3072), (500, 768, 64), (302, 40, 192)])
 def test_gemm_bt(k, m, n, k_):
     print("gemm_bt", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_)
@@ -379,7 +382,7 @@ def test_gemm_bt(k, m, n, k_):
     got = k.gemm_bt(dev(a), bt).cpu().numpy()
     # the same rows through the untransposed kernel: both accumulate k in the same order
     assert np.array_equal(got, k.gemm(dev(a), dev(b)).cpu().numpy())
-    rows = np.unique(np.concatenate([np.arange(0, 300), np.arange(m - 300, m), rng.randint(0, m, 400)]))
+    rows = np.unique(np.concatenate([np.arange(0, min(m, 300)), np.arange(max(m - 300, 0), m), rng.randint(0, m, 400)]))
     exact = a[rows].astype(np.float64) @ b.astype(np.float64)
     assert np.all(np.abs(got[rows].astype(np.float64) - exact) <= 0.51 * half_ulp(exact) + 1e-5 * np.abs(exact).max())
     gotb = k.gemm_bt(dev(a), bt, bias=dev(bias)).cpu().numpy()
@@ -391,7 +394,8 @@ def test_gemm_bt(k, m, n, k_):
 
 # A sequence gives the same bits in a batch of any size: every fp16 kernel accumulates k in the same order, so the
 # rows of a small problem (64x128 tiles), a middle one (128x256 tiles) and a large one (persistent 256x256 tiles, B in
-# either storage order) agree bit for bit; the two fp32 tiles likewise.
+# either storage order) agree bit for bit, and so do the four one-tile-per-workgroup kernels for k-contiguous B
+# (128x128, 64x128, 64x64, 32x64); the two fp32 tiles likewise.
 @pytest.mark.parametrize("n,k_", [(768, 768), (768, 3072), (3072, 768)])
 def test_gemm_same_bits_in_every_kernel(k, n, k_):
     print("gemm same bits", n, k_, flush=True)
@@ -400,9 +404,13 @@ def test_gemm_same_bits_in_every_kernel(k, n, k_):
     a = dev(o.rnd(rng.randn(m, k_), "fp16"))
     b = dev(o.rnd(0.05 * rng.randn(k_, n), "fp16"))
     big = k.gemm(a, b).cpu().numpy()
-    assert np.array_equal(k.gemm_bt(a, k.transpose_weight(b)).cpu().numpy(), big)
+    bt = k.transpose_weight(b)
+    assert np.array_equal(k.gemm_bt(a, bt).cpu().numpy(), big)
     for rows in (6000, 2500, 300, 1):
         part = k.gemm(a[:rows].contiguous(), b).cpu().numpy()
+        assert np.array_equal(part, big[:rows]), rows
+    for rows in (9000, 6000, 4000, 2000, 1000, 500, 130, 1):
+        part = k.gemm_bt(a[:rows].contiguous(), bt).cpu().numpy()
         assert np.array_equal(part, big[:rows]), rows
     a32, b32 = a.float(), b.float()
     big32 = k.gemm(a32, b32).cpu().numpy()
@@ -430,7 +438,8 @@ def test_gemm_bias_gelu_equals_the_two_passes(k, dtype, m, n, k_):
         k.gemm(dev(a), dev(b), gelu=True)
 
 
-@pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (5000, 3072, 768)])
+@pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (5000, 3072, 768), (2000, 3072, 768),
+                                    (1000, 776, 128), (400, 768, 768), (350, 200, 64)])
 def test_gemm_bt_bias_gelu_equals_the_two_passes(k, m, n, k_):
     print("gemm_bt_bias_gelu", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_ + 1)
@@ -452,8 +461,8 @@ def test_gemm_bt_bias_gelu_equals_the_two_passes(k, m, n, k_):
         k.gemm_bt(dev(a), bt, gelu=True)
 
 
-def test_gemm_bt_small_shapes_are_refused(k):
-    a = torch.zeros(1000, 768, dtype=torch.float16, device="cuda")
-    bt = torch.zeros(768, 768, dtype=torch.float16, device="cuda")
-    with pytest.raises(Exception, match="128 tiles"):
+def test_gemm_bt_refuses_k_that_is_no_multiple_of_64(k):
+    a = torch.zeros(1000, 96, dtype=torch.float16, device="cuda")
+    bt = torch.zeros(768, 96, dtype=torch.float16, device="cuda")
+    with pytest.raises(Exception, match="k % 64"):
         k.gemm_bt(a, bt)
