@@ -139,7 +139,8 @@ LayerWs layer_ws(et_dtype dtype, int B, int S, int heads, int d) {
   w.qkv = off;   off += align_up(rows * 3 * H * e, 256);
   w.ctx = off;   off += align_up(rows * H * e, 256);
   w.attn = off;  off += align_up(rows * H * e, 256);
-  w.inter = off; off += align_up(rows * 4 * H * e, 256);
+  // whole tiles of 256 rows: the FFN's intermediate may be handed over in blocks of [256 rows][64 columns]
+  w.inter = off; off += align_up(align_up(rows, 256) * 4 * H * e, 256);
   w.seq = off;   off += align_up(et::seq_table_words(B) * sizeof(int32_t), 256);
   // fp16: k-contiguous copies of the six dense kernels (3 H^2 + H^2 + 4 H^2 + 4 H^2 elements) for the large-M GEMM
   w.wt = off;    off += dtype == ET_FP16 ? align_up(12 * H * H * e, 256) : 0;
@@ -491,13 +492,18 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   g1.b_transposed = t_up;
   // bias + GELU are applied to each tile on its way out of the GEMM: no pass of its own over [T,4H]
   g1.bias[0] = w->inter_bias; g1.gelu = true;
+  // where both FFN projections run the persistent k-contiguous kernel, [T,4H] goes from one to the other in blocks
+  const bool blocked = t_up && t_down && et::gemm_blocked_handover(dt, rows, F, H);
+  g1.c_blocked = blocked;
   et::launch_gemm(dt, g1, inter, F, rows, F, H, T, st);
-  g1.bias[0] = nullptr; g1.gelu = false;
+  g1.bias[0] = nullptr; g1.gelu = false; g1.c_blocked = false;
   if ((s = check_launch(h, "FFN up")) != ET_OK) return s;
   // FFN down + bias + residual(LN1 output) + LayerNorm (:229-247)
   g1.A[0] = inter; g1.B[0] = t_down ? wt_down : w->output_kernel;
   g1.b_transposed = t_down;
+  g1.a_blocked = blocked;
   et::launch_gemm(dt, g1, out, H, rows, H, F, T, st);
+  g1.a_blocked = false;
   et::launch_bias_residual_layernorm(dt, out, attn, w->output_bias, w->output_layernorm_gamma,
                                      w->output_layernorm_beta, rows, H, T, st);
   if ((s = check_launch(h, "FFN down")) != ET_OK) return s;

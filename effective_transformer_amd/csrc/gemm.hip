@@ -37,6 +37,8 @@ struct GemmArgs {
   int per_xcd;               // workgroups per XCD slot of the launch
   int reverse_walk = 0;      // persistent kernel: walk the tiles from the last one
   int gelu = 0;              // C = gelu(A.B + bias) instead of A.B + bias (bias must be set)
+  int a_blocked = 0;         // pair kernel: A / C hold every tile of 256 rows as blocks of [256 rows][64 columns]
+  int c_blocked = 0;         //   (see GemmGroups)
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -589,8 +591,10 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
     t.grp = tn_all / args.tiles_n;
     t.m0 = tm * kPBM;
     t.n0 = (tn_all - t.grp * args.tiles_n) * kPBN;
+    // a blocked A holds whole tiles: rows beyond the valid count are there (written by the producer from zero rows)
     t.a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<_Float16*>((const _Float16*)args.A[t.grp] + (size_t)t.m0 * K), 0, min(rows - t.m0, kPBM) * K * 2, 0x00020000);
+        const_cast<_Float16*>((const _Float16*)args.A[t.grp] + (size_t)t.m0 * K), 0,
+        (args.a_blocked ? kPBM : min(rows - t.m0, kPBM)) * K * 2, 0x00020000);
     t.b = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16*>((const _Float16*)args.B[t.grp] + (size_t)t.n0 * K), 0, min(N - t.n0, kPBN) * K * 2, 0x00020000);
     return t;
@@ -604,15 +608,19 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
   for (int j = 0; j < 4; ++j) {
     const int row = wave * 32 + j * 8 + (lane >> 3);
     const int c = (lane & 7) ^ pair_swizzle(row);
-    voff_a[j] = ((uint32_t)row * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+    // blocked A: the 128 bytes of a row and pair lie 128 bytes from the next row's, a pair is one block of 32 KB
+    voff_a[j] = args.a_blocked ? (uint32_t)row * 128u + (uint32_t)c * 16u
+                               : ((uint32_t)row * (uint32_t)K + (uint32_t)c * 8u) * 2u;
     const int col = (row & ~63) + (row & 15) * 4 + ((row >> 4) & 3);
     voff_b[j] = ((uint32_t)col * (uint32_t)K + (uint32_t)c * 8u) * 2u;
   }
+  const int a_pair_bytes = args.a_blocked ? kQAPair : 128;       // from one pair of k-steps of A to the next
   // instruction q (0..3: A, 4..7: B^T) of this wave's share of pair `pr` of a tile into slot `slot`
   auto issue1 = [&](int slot, int pr, const __amdgpu_buffer_rsrc_t& ra, const __amdgpu_buffer_rsrc_t& rb, int q) {
     unsigned char* st = smem + slot * kQPair;
     if (q < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, ET_LDS_PTR(st + (wave * 4 + q) * 1024), 16, voff_a[q], pr * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, ET_LDS_PTR(st + (wave * 4 + q) * 1024), 16, voff_a[q],
+                                               pr * a_pair_bytes, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, ET_LDS_PTR(st + kQAPair + (wave * 4 + q - 4) * 1024), 16,
                                                voff_b[q - 4], pr * 128, 0, 0);
@@ -731,11 +739,17 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
       const int col = cur.n0 + wn * 64 + l16 * 4;
       if (col < N) {
         const int tile_rows = min(rows - cur.m0, kPBM), tile_cols = min(N - cur.n0, kPBN);
-        _Float16* cbase = (_Float16*)args.C + (size_t)cur.m0 * args.ldc + (size_t)cur.grp * N + cur.n0;
-        const __amdgpu_buffer_rsrc_t rc =
-            __builtin_amdgcn_make_buffer_rsrc(cbase, 0, ((tile_rows - 1) * args.ldc + tile_cols) * 2, 0x00020000);
-        const uint32_t row_bytes = (uint32_t)args.ldc * 2u;
-        uint32_t voff = ((uint32_t)(wm * 128 + g * 4) * (uint32_t)args.ldc + (uint32_t)(wn * 64 + l16 * 4)) * 2u;
+        // Blocked C (one group, n a multiple of 256, whole tiles of rows allocated): the tile's four 64-column blocks
+        // of [256 rows][128 bytes] follow each other; rows beyond the valid count are written too (gelu(bias) of zero
+        // rows), so that a consumer may read whole tiles.
+        _Float16* cbase = args.c_blocked ? (_Float16*)args.C + (size_t)cur.m0 * args.ldc + (size_t)cur.n0 * kPBM
+                                         : (_Float16*)args.C + (size_t)cur.m0 * args.ldc + (size_t)cur.grp * N + cur.n0;
+        const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(
+            cbase, 0, args.c_blocked ? kPBM * kPBN * 2 : ((tile_rows - 1) * args.ldc + tile_cols) * 2, 0x00020000);
+        const uint32_t row_bytes = args.c_blocked ? 128u : (uint32_t)args.ldc * 2u;
+        uint32_t voff = args.c_blocked
+                            ? (uint32_t)wn * (uint32_t)kQAPair + (uint32_t)(wm * 128 + g * 4) * 128u + (uint32_t)l16 * 8u
+                            : ((uint32_t)(wm * 128 + g * 4) * (uint32_t)args.ldc + (uint32_t)(wn * 64 + l16 * 4)) * 2u;
         // the offset is the same for every tile; the empty asm keeps the compiler from computing all 32 store offsets
         // once and holding them in registers across the k loop
         asm volatile("" : "+v"(voff));
@@ -1217,6 +1231,12 @@ bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int gr
 // Inside the layer the transposed copy pays off for the wide projections (QKV, FFN up: many column tiles re-read a
 // short k extent).  With k >= n the activations stream through L2 once per few tiles and the [k][n] kernel, whose B rows
 // are 512 contiguous bytes, is as fast inside the layer as the k-contiguous one is on its own, so the copy is skipped.
+bool gemm_blocked_handover(DType t, int m_bound, int wide, int narrow) {
+  return gemm_takes_transposed_b(t, m_bound, wide, wide, narrow, 1) && use_persistent(m_bound, wide, wide, narrow, 1) &&
+         gemm_takes_transposed_b(t, m_bound, narrow, narrow, wide, 1) && use_persistent(m_bound, narrow, narrow, wide, 1) &&
+         wide % kPBN == 0 && (uint64_t)((m_bound + kPBM - 1) / kPBM * kPBM) * (uint64_t)wide * 2u <= 0xffffffffull;
+}
+
 bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
   return gemm_takes_transposed_b(t, m_bound, ldc, n, k, groups) && use_persistent(m_bound, ldc, n, k, groups) &&
          (long)n * groups >= 2L * k;
@@ -1261,6 +1281,8 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.k = k;
   a.groups = g.groups;
   a.gelu = g.gelu ? 1 : 0;
+  a.a_blocked = g.a_blocked ? 1 : 0;
+  a.c_blocked = g.c_blocked ? 1 : 0;
   if (t == DType::F16) {
     if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
       launch_f16_persistent(a, stream, g.b_transposed);

@@ -96,8 +96,17 @@ struct GemmGroups {
   // C = gelu(A.B + bias): bias + GELU as in launch_bias_gelu, same rounding points, applied to each tile on its way
   // out; bias[g] must be set
   bool gelu = false;
+  // Hand-over of a wide intermediate between two launches of the persistent k-contiguous kernel (the FFN's [T, 4H]
+  // matrix): the producer writes C, the consumer reads A, with every tile of 256 rows stored as consecutive blocks of
+  // [256 rows][64 columns] (32 KB each) instead of row-major, so that the consumer's operand fetches, 128 bytes per row
+  // and pair of k-steps, are contiguous in memory instead of one row stride apart.  Only where
+  // gemm_blocked_handover() says so; the matrix must be allocated for a whole number of 256-row tiles.
+  bool c_blocked = false, a_blocked = false;
 };
 bool gemm_supported(DType t, int n, int k, int groups);
+// True when both C = A.B1 ([m, wide] from k = narrow) and the product that consumes it (k = wide, n = narrow) run the
+// persistent k-contiguous kernel, given k-contiguous copies of both weights.
+bool gemm_blocked_handover(DType t, int m_bound, int wide, int narrow);
 // The large-M fp16 kernel is faster when B comes k-contiguous ([n][k]): both operands then reach the
 // MFMA with 128-bit LDS reads and no register transpose.  True when launch_gemm would use that kernel.
 bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
