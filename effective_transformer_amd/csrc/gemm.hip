@@ -542,21 +542,26 @@ constexpr int kQSmem = 2 * kQPair;
 
 __device__ __forceinline__ int pair_swizzle(int row) { return (row >> 1) & 7; }
 
-template <bool GELU>
+// MI: 16-row blocks per wave, i.e. tiles of 32 MI rows (256, 224, 192 or 160).  The tile count of a launch rarely
+// fills whole rounds of the chip; a lower tile can turn "one round and a bit" into one round (launch_f16_persistent
+// chooses).  The A part of an LDS slot keeps its 256 rows; the rows beyond the tile lie outside the tile's buffer
+// descriptor and cost no traffic.
+template <bool GELU, int MI>
 __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // 0..7, scalar
-  const int wm = wave & 1, wn = (wave >> 1) & 3;                  // 128-row half, 64-column quarter of the tile
+  constexpr int BM = 32 * MI;                                     // rows of a tile
+  const int wm = wave & 1, wn = (wave >> 1) & 3;                  // (16 MI)-row half, 64-column quarter of the tile
   const int l16 = lane & 15, g = lane >> 4;
   const int N = args.n, K = args.k;
   const int np = K / 64;                                          // pairs of k-steps per tile, >= 2
 
   const int rows = args.rows_dev ? min(*args.rows_dev, args.m_bound) : args.m_bound;
   const int tiles_n_all = args.tiles_n * args.groups;
-  const int total = ((rows + kPBM - 1) / kPBM) * tiles_n_all;     // tiles that hold valid rows (a prefix in tile order)
+  const int total = ((rows + BM - 1) / BM) * tiles_n_all;     // tiles that hold valid rows (a prefix in tile order)
   const int per_xcd = (total + kXcds - 1) / kXcds;
   const int xcd = blockIdx.x % kXcds;
   const int G = gridDim.x;                                        // multiple of 8
@@ -589,12 +594,12 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
     const int tm = tile / tiles_n_all;
     const int tn_all = tile - tm * tiles_n_all;
     t.grp = tn_all / args.tiles_n;
-    t.m0 = tm * kPBM;
+    t.m0 = tm * BM;
     t.n0 = (tn_all - t.grp * args.tiles_n) * kPBN;
     // a blocked A holds whole tiles: rows beyond the valid count are there (written by the producer from zero rows)
     t.a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16*>((const _Float16*)args.A[t.grp] + (size_t)t.m0 * K), 0,
-        (args.a_blocked ? kPBM : min(rows - t.m0, kPBM)) * K * 2, 0x00020000);
+        (args.a_blocked ? BM : min(rows - t.m0, BM)) * K * 2, 0x00020000);
     t.b = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16*>((const _Float16*)args.B[t.grp] + (size_t)t.n0 * K), 0, min(N - t.n0, kPBN) * K * 2, 0x00020000);
     return t;
@@ -628,7 +633,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
 
   // operand reads: row (wm*128 + i*16 + l16) resp. (wn*64 + j*16 + l16), chunk (4*half + g), swizzled
   const int sw = pair_swizzle(l16);
-  const int a_rd[2] = {(wm * 128 + l16) * 128 + ((g ^ sw) * 16), (wm * 128 + l16) * 128 + (((4 + g) ^ sw) * 16)};
+  const int a_rd[2] = {(wm * 16 * MI + l16) * 128 + ((g ^ sw) * 16), (wm * 16 * MI + l16) * 128 + (((4 + g) ^ sw) * 16)};
   const int b_rd[2] = {kQAPair + (wn * 64 + l16) * 128 + ((g ^ sw) * 16),
                        kQAPair + (wn * 64 + l16) * 128 + (((4 + g) ^ sw) * 16)};
 
@@ -649,8 +654,8 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
   }
   Src cur = locate(idx), nxt = cur;
 
-  float4v acc[8][4];
-  half8 a[2][8], b[2][4];
+  float4v acc[MI][4];
+  half8 a[2][MI], b[2][4];
   int pairs_done = 0;                            // by this workgroup: slot of a pair = pairs_done & 1
 
   // One k-step: MFMAs on operand set P; half `rh` of slot `rs` is read into the other set; with DMA set, this wave's
@@ -663,19 +668,22 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
     constexpr int rh = 1 - P;                    // the even step reads half 1 of its own pair, the odd step half 0 of the next
     const unsigned char* ns = smem + rs * kQPair;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (i < 2) {
-        b[1 - P][2 * i] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + (2 * i) * 2048);
-        b[1 - P][2 * i + 1] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + (2 * i + 1) * 2048);
-      } else if (i < 6) {
-        a[1 - P][2 * (i - 2)] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (2 * (i - 2)) * 2048);
-        a[1 - P][2 * (i - 2) + 1] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (2 * (i - 2) + 1) * 2048);
+    for (int i = 0; i < MI; ++i) {
+      // two of the 4 + MI operand reads of the next step in front of each group of four MFMAs (B^T blocks first)
+#pragma unroll
+      for (int r = 2 * i; r < 2 * i + 2 && r < 4 + MI; ++r) {
+        if (r < 4) b[1 - P][r] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + r * 2048);
+        else a[1 - P][r - 4] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (r - 4) * 2048);
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[P][i], b[P][j],
                                                            FIRST ? float4v{0.f, 0.f, 0.f, 0.f} : acc[i][j], 0, 0, 0);
-      if (DMA) issue1(ds, dpr, da, db, i);
+      if (DMA) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+          if (q * MI / 8 == i) issue1(ds, dpr, da, db, q);      // the eight DMA instructions spread over the MI groups
+      }
       __builtin_amdgcn_sched_barrier(0);         // keeps the reads and the DMA where they are between the MFMA groups
     }
   };
@@ -692,7 +700,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
 #pragma unroll
   for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const half8*>(smem + b_rd[0] + j * 2048);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) a[0][i] = *reinterpret_cast<const half8*>(smem + a_rd[0] + i * 2048);
+  for (int i = 0; i < MI; ++i) a[0][i] = *reinterpret_cast<const half8*>(smem + a_rd[0] + i * 2048);
 
   bool first_tile = true;
   while (true) {
@@ -738,7 +746,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
       // bounds check, and the only per-store address arithmetic is one add on the running byte offset
       const int col = cur.n0 + wn * 64 + l16 * 4;
       if (col < N) {
-        const int tile_rows = min(rows - cur.m0, kPBM), tile_cols = min(N - cur.n0, kPBN);
+        const int tile_rows = min(rows - cur.m0, BM), tile_cols = min(N - cur.n0, kPBN);
         // Blocked C (one group, n a multiple of 256, whole tiles of rows allocated): the tile's four 64-column blocks
         // of [256 rows][128 bytes] follow each other; rows beyond the valid count are written too (gelu(bias) of zero
         // rows), so that a consumer may read whole tiles.
@@ -748,8 +756,8 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
             cbase, 0, args.c_blocked ? kPBM * kPBN * 2 : ((tile_rows - 1) * args.ldc + tile_cols) * 2, 0x00020000);
         const uint32_t row_bytes = args.c_blocked ? 128u : (uint32_t)args.ldc * 2u;
         uint32_t voff = args.c_blocked
-                            ? (uint32_t)wn * (uint32_t)kQAPair + (uint32_t)(wm * 128 + g * 4) * 128u + (uint32_t)l16 * 8u
-                            : ((uint32_t)(wm * 128 + g * 4) * (uint32_t)args.ldc + (uint32_t)(wn * 64 + l16 * 4)) * 2u;
+                            ? (uint32_t)wn * (uint32_t)kQAPair + (uint32_t)(wm * 16 * MI + g * 4) * 128u + (uint32_t)l16 * 8u
+                            : ((uint32_t)(wm * 16 * MI + g * 4) * (uint32_t)args.ldc + (uint32_t)(wn * 64 + l16 * 4)) * 2u;
         // the offset is the same for every tile; the empty asm keeps the compiler from computing all 32 store offsets
         // once and holding them in registers across the k loop
         asm volatile("" : "+v"(voff));
@@ -758,7 +766,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
         half4 bias4 = {(_Float16)-0.0f, (_Float16)-0.0f, (_Float16)-0.0f, (_Float16)-0.0f};
         if (args.bias[cur.grp] != nullptr) bias4 = *reinterpret_cast<const half4*>((const _Float16*)args.bias[cur.grp] + col);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < MI; ++i) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             half4 o;
@@ -1148,11 +1156,51 @@ int device_cu_count() {
   return n;
 }
 
+// Rows per tile of the k-contiguous persistent kernel, as the count MI of 16-row blocks per wave (tile = 32 MI rows).
+// A launch takes rounds x tile time, and the last round of a band of tiles (one XCD, cus / 8 workgroups) is often far
+// from full; a lower tile can then do with fewer rounds, or with a shorter single round: 13097 rows x 768 columns are
+// 156 tiles of 256 rows, one round on 61 % of the CUs, or 246 tiles of 160 rows, one round on 96 % of them.  The time
+// of a tile falls much more slowly than its height (the B^T half of the operand stream, the DMA and the LDS traffic
+// stay): measured about 1.45 us per pair of k-steps at 256 rows and 1.3 us at 160, i.e. proportional to MI + 21.  A
+// lower tile must win 3 % by that estimate (measured: FFN-down of 13097 rows 75 -> 64 us, of 15866 rows 76 -> 70 us,
+// attention-out 26 -> 24 us; the 13097 x 1024 one of BERT-large 35 -> 31.5 us; all with the same bits).
+int pair_kernel_row_blocks(int m_bound, int n, int groups) {
+  const int cus = device_cu_count();
+  const int wgs = std::max(1, cus / kXcds);
+  const int tiles_n = (n + kPBN - 1) / kPBN * groups;
+  auto cost = [&](int mi) {
+    const long tiles = (long)((m_bound + 32 * mi - 1) / (32 * mi)) * tiles_n;
+    const long n_loc = (tiles + kXcds - 1) / kXcds;
+    const long full = n_loc / wgs, rem = n_loc % wgs;
+    // a rest of at most half the workgroups is shared, two workgroups per tile
+    const double rounds = (double)full + (rem == 0 ? 0.0 : (2 * rem <= wgs ? 0.55 : 1.0));
+    return rounds * (mi + 21);
+  };
+  const double cost8 = cost(8);
+  double best = cost8;
+  int best_mi = 8;
+  for (int mi = 7; mi >= 5; --mi) {
+    const double c = cost(mi);
+    if (c < 0.97 * cost8 && c < best) {
+      best = c;
+      best_mi = mi;
+    }
+  }
+  return best_mi;
+}
+
+template <bool GELU, int MI>
+void launch_pair(const GemmArgs& a, int grid, hipStream_t stream) {
+  auto kern = gemm_f16_pair_kernel<GELU, MI>;
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), kQSmem);
+  kern<<<grid, kPThreads, kQSmem, stream>>>(a);
+}
+
 void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
-  if (b_transposed && a.gelu) allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_pair_kernel<true>), kQSmem);
-  else if (b_transposed) allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_pair_kernel<false>), kQSmem);
-  else allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel), kPSmem);
-  a.tiles_m = (a.m_bound + kPBM - 1) / kPBM;
+  // the blocked hand-over is laid out for tiles of 256 rows
+  const int mi = !b_transposed || a.a_blocked || a.c_blocked ? 8 : pair_kernel_row_blocks(a.m_bound, a.n, a.groups);
+  const int bm = 32 * mi;
+  a.tiles_m = (a.m_bound + bm - 1) / bm;
   a.tiles_n = (a.n + kPBN - 1) / kPBN;
   const int total = a.tiles_m * a.tiles_n * a.groups;
   int grid = std::min(device_cu_count(), total);
@@ -1161,9 +1209,23 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
   // k > n: A is the big operand and was written front to back by the kernel before this one, so its last rows are the
   // ones most likely still in the last-level cache: walk the tiles from the end
   a.reverse_walk = a.k > a.n ? 1 : 0;
-  if (b_transposed && a.gelu) gemm_f16_pair_kernel<true><<<grid, kPThreads, kQSmem, stream>>>(a);
-  else if (b_transposed) gemm_f16_pair_kernel<false><<<grid, kPThreads, kQSmem, stream>>>(a);
-  else gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
+  if (!b_transposed) {
+    allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel), kPSmem);
+    gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
+    return;
+  }
+#define ET_PAIR_CASE(M)                                  \
+  case M:                                                \
+    if (a.gelu) launch_pair<true, M>(a, grid, stream);   \
+    else launch_pair<false, M>(a, grid, stream);         \
+    break;
+  switch (mi) {
+    ET_PAIR_CASE(8)
+    ET_PAIR_CASE(7)
+    ET_PAIR_CASE(6)
+    ET_PAIR_CASE(5)
+  }
+#undef ET_PAIR_CASE
 }
 
 // few big tiles would leave most of the 256 CUs idle: the persistent 256x256 kernel only runs when there is work
@@ -1232,8 +1294,10 @@ bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int gr
 // short k extent).  With k >= n the activations stream through L2 once per few tiles and the [k][n] kernel, whose B rows
 // are 512 contiguous bytes, is as fast inside the layer as the k-contiguous one is on its own, so the copy is skipped.
 bool gemm_blocked_handover(DType t, int m_bound, int wide, int narrow) {
+  // ... and both would run on tiles of 256 rows anyway (a lower tile for one of them is worth more than the hand-over)
   return gemm_takes_transposed_b(t, m_bound, wide, wide, narrow, 1) && use_persistent(m_bound, wide, wide, narrow, 1) &&
          gemm_takes_transposed_b(t, m_bound, narrow, narrow, wide, 1) && use_persistent(m_bound, narrow, narrow, wide, 1) &&
+         pair_kernel_row_blocks(m_bound, wide, 1) == 8 && pair_kernel_row_blocks(m_bound, narrow, 1) == 8 &&
          wide % kPBN == 0 && (uint64_t)((m_bound + kPBM - 1) / kPBM * kPBM) * (uint64_t)wide * 2u <= 0xffffffffull;
 }
 

@@ -364,11 +364,13 @@ def test_gemm(k, dtype, m, n, k_):
 
 # The k-contiguous-B kernels: the persistent 256x256 one from 128 such tiles on (first six shapes; the last two of
 # those leave a last round that keeps at most half of the workgroups busy, so those tiles are shared by two
-# workgroups, one per 128-column half, one of them with a ragged last column tile), below that one tile per workgroup
+# workgroups, one per 128-column half, one of them with a ragged last column tile; the next three run on tiles of
+# 160, 192 and 224 rows, which fill the chip's single round better), below that one tile per workgroup
 # of 128x128 (one or two workgroups per CU), 64x128, 64x64 or 32x64, with ragged last tiles in both directions and a
 # single pair of k-steps.  The oracle product is taken on the CPU in float64 for a sample of rows.
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072),
                                     (23301, 768, 768), (14000, 1032, 128),
+                                    (13097, 768, 3072), (15866, 768, 768), (13097, 1024, 1024),
                                     (6000, 776, 768), (4000, 768, 3072), (3000, 1032, 128), (2000, 768, 768),
                                     (1001, 776, 3072), (500, 768, 64), (302, 40, 192)])
 def test_gemm_bt(k, m, n, k_):
