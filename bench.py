@@ -109,6 +109,30 @@ def _time_kernel(fn, iters, warm=3):
     return s.elapsed_time(e) / iters          # ms per launch
 
 
+def mfma_ceiling(iters=4000):
+    """The MFMA rate this GPU sustains under the instruction mix of the large fp16 GEMM's inner loop (MFMAs + LDS
+    operand reads, no global memory), with zero and with random operands: et_calibrate_mfma, timed with HIP events.
+    Switching activity costs clock, so the rate on random data, not the data-sheet peak, is the ceiling the GEMMs run
+    under on this part."""
+    import ctypes as C
+    import torch
+    from effective_transformer_amd import _lib, ops
+    lib = _lib.load()
+    h = ops.handle(torch.device("cuda:0"))
+    sink = torch.empty(lib.et_calibrate_mfma_sink_bytes(h), dtype=torch.uint8, device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    fl = C.c_double(0.0)
+    out = {}
+    for name, rnd in (("zero_operands", 0), ("random_operands", 1)):
+        def run():
+            _lib.check(lib.et_calibrate_mfma(h, rnd, iters, C.c_void_p(sink.data_ptr()), sink.numel(), C.byref(fl), st), h)
+        ms = min(_time_kernel(run, 5, warm=2) for _ in range(2))
+        out[name + "_tflops"] = round(fl.value / ms / 1e9, 1)
+    out["unit"] = "TFLOP/s"
+    out["what"] = "8 waves per CU, per wave and k-step 32 v_mfma_f32_16x16x32_f16 + 12 ds_read_b128, no global memory"
+    return out
+
+
 def per_kernel(wl, T, mask_np, iters=20, vendor_gemm=False):
     """Times every kernel of the path in isolation at the workload's real shapes and prices it
     against its roofline with ALGORITHMIC bytes / flops.  vendor_gemm: also time the vendor library's GEMM
@@ -354,6 +378,8 @@ def main():
     ap.add_argument("--cpu-seqs", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--calibrate-mfma", action="store_true",
+                    help="also measure the MFMA rate the GPU sustains on zero and on random operands (fp16)")
     ap.add_argument("--calibrate-gemm", action="store_true",
                     help="also time the vendor library's GEMM (torch.matmul) on the four projection shapes")
     ap.add_argument("--fold-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
@@ -449,6 +475,14 @@ def main():
                     "unit": kd["unit"], "frac": kd["frac_in_layer"], "ms": kd["ms_in_layer"],
                     "measured": "HIP events around the kernel inside the layer's launch sequence, %d launches" % (4 * wl.layers),
                     "alone": alone, "traffic": measured_traffic(wl.name, dom)}
+    ceiling = None
+    if a.calibrate_mfma:
+        try:
+            ceiling = mfma_ceiling()
+            if roof is not None and roof["bound"] == "mfma" and wl.dtype == "fp16":
+                roof["frac_of_sustained_on_random_operands"] = round(roof["achieved"] / ceiling["random_operands_tflops"], 4)
+        except Exception as ex:      # a failed calibration must not take the benchmark line down
+            ceiling = {"error": str(ex)[:200]}
     cpu = None
     if not a.no_cpu:
         cpu = cpu_baseline(w, a.cpu_seqs)
@@ -466,7 +500,7 @@ def main():
                                % (wl.name, wl.layers, wl.H, wl.heads, wl.d, wl.F, wl.B, wl.S, T),
                    "valid_tokens": T, "padded_tokens": wl.B * wl.S},
         "roofline": roof, "layer_ms_sum_of_kernels": None if layer_sum is None else round(layer_sum, 4),
-        "kernels": kernels, "cpu_baseline": cpu,
+        "kernels": kernels, "cpu_baseline": cpu, "mfma_ceiling": ceiling,
     }))
 
 

@@ -86,6 +86,8 @@ SIGNATURES = {
     "et_transpose_weight": (_i, [_vp, _i, _vp, _vp, _i, _i, _vp]),
     "et_gemm_bt": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_gemm_bt_bias_gelu": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "et_calibrate_mfma_sink_bytes": (_sz, [_vp]),
+    "et_calibrate_mfma": (_i, [_vp, _i, _i, _vp, _sz, C.POINTER(C.c_double), _vp]),
 }
 
 _lib = None

@@ -800,4 +800,33 @@ et_status et_gemm_bt_bias_gelu(et_handle h, et_dtype dtype, const void* A, const
   return gemm_bt_impl(h, dtype, A, Bt, C, bias, m, n, k, m_dev, stream, true, "et_gemm_bt_bias_gelu");
 }
 
+namespace {
+int current_cu_count() {
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount <= 0)
+    return 256;
+  return prop.multiProcessorCount;
+}
+}  // namespace
+
+size_t et_calibrate_mfma_sink_bytes(et_handle h) {
+  Entry entry(h);
+  if (entry.status != ET_OK) return 0;
+  return et::mfma_ceiling_sink_bytes(current_cu_count());
+}
+
+et_status et_calibrate_mfma(et_handle h, int random_operands, int iters, void* sink, size_t sink_bytes, double* flops,
+                            void* stream) {
+  Entry entry(h);
+  et_status s = entry.status;
+  if (s != ET_OK) return s;
+  ET_REQUIRE(h, sink && flops, "null pointer");
+  ET_REQUIRE(h, iters >= 1 && iters <= (1 << 22), "iters must be in 1 .. 4194304");
+  const int cus = current_cu_count();
+  if (sink_bytes < et::mfma_ceiling_sink_bytes(cus)) return fail(h, ET_WORKSPACE_TOO_SMALL, "sink buffer too small");
+  *flops = et::launch_mfma_ceiling(random_operands != 0, cus, iters, (float*)sink, (hipStream_t)stream);
+  return check_launch(h, "MFMA calibration");
+}
+
 }  // extern "C"

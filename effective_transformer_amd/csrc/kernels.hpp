@@ -133,4 +133,11 @@ void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, con
 void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k,
                  const int32_t* rows_dev, hipStream_t stream);
 
+// ---- calibrate.hip: measurement aid ---------------------------------------------------------------------
+// One launch of `iters` k-steps of the large fp16 GEMM's inner loop (MFMAs + LDS operand reads, no global memory) on
+// `cus` workgroups of 8 wavefronts, with zero or random operands; returns the floating-point operations of the launch.
+// `sink` receives one float per thread (mfma_ceiling_sink_bytes).
+size_t mfma_ceiling_sink_bytes(int cus);
+double launch_mfma_ceiling(bool random_operands, int cus, int iters, float* sink, hipStream_t stream);
+
 }  // namespace et

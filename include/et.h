@@ -317,6 +317,17 @@ et_status et_gemm_bt(et_handle h, et_dtype dtype, const void* A, const void* Bt,
 et_status et_gemm_bt_bias_gelu(et_handle h, et_dtype dtype, const void* A, const void* Bt, void* C, const void* bias,
                                int m, int n, int k, const int32_t* m_dev, void* stream);
 
+/* Measurement aid, no counterpart in the reference and no part of the encoder path: one launch of `iters` k-steps of
+ * the large fp16 GEMM's inner loop (per wavefront 32 v_mfma_f32_16x16x32_f16 and 12 16-byte LDS operand reads, 8
+ * wavefronts on every CU, no global memory traffic) with operands that are all zero (random_operands == 0) or random
+ * halves.  *flops receives the floating-point operations of the launch; the caller times it with events on `stream`.
+ * The rate with random operands is the ceiling a GEMM on real data runs under on this part (switching activity costs
+ * clock), which is what bench.py --calibrate-mfma reports beside the data-sheet peak.  `sink` is a device buffer of
+ * et_calibrate_mfma_sink_bytes() bytes that receives one float per thread. */
+size_t et_calibrate_mfma_sink_bytes(et_handle h);
+et_status et_calibrate_mfma(et_handle h, int random_operands, int iters, void* sink, size_t sink_bytes, double* flops,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif

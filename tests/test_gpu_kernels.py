@@ -468,3 +468,26 @@ def test_gemm_bt_refuses_k_that_is_no_multiple_of_64(k):
     bt = torch.zeros(768, 96, dtype=torch.float16, device="cuda")
     with pytest.raises(Exception, match="k % 64"):
         k.gemm_bt(a, bt)
+
+
+# The measurement aid: a launch returns its floating-point operation count (CUs x 8 waves x iters x 64 MFMAs x 16384),
+# fills the sink with finite sums (zero for zero operands) and refuses a sink that is too small.
+def test_calibrate_mfma(ops):
+    import ctypes as C
+    from effective_transformer_amd import _lib
+    lib = _lib.load()
+    h = ops.handle(torch.device("cuda:0"))
+    nbytes = lib.et_calibrate_mfma_sink_bytes(h)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert nbytes == cus * 512 * 4
+    sink = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    fl = C.c_double(0.0)
+    for rnd in (0, 1):
+        _lib.check(lib.et_calibrate_mfma(h, rnd, 10, C.c_void_p(sink.data_ptr()), nbytes, C.byref(fl), st), h)
+        torch.cuda.synchronize()
+        assert fl.value == cus * 8 * 10 * 64 * 16384.0
+        assert bool(torch.isfinite(sink).all())
+        assert bool((sink == 0).all()) == (rnd == 0)
+    assert lib.et_calibrate_mfma(h, 0, 10, C.c_void_p(sink.data_ptr()), nbytes - 4, C.byref(fl), st) == 2   # ET_WORKSPACE_TOO_SMALL
+    assert lib.et_calibrate_mfma(h, 0, 0, C.c_void_p(sink.data_ptr()), nbytes, C.byref(fl), st) == 1         # ET_INVALID_ARGUMENT
