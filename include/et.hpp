@@ -102,9 +102,18 @@ class Encoder {
     check_hip(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
   }
 
+  ~Encoder() {
+    if (host_count_) (void)hipHostFree(host_count_);
+    if (copied_) (void)hipEventDestroy(copied_);
+  }
+  Encoder(const Encoder&) = delete;
+  Encoder& operator=(const Encoder&) = delete;
+
   // from_tensor [B,S,H], mask int32 [B,S], attr_mask [B,S,S] in dtype -> out [B,S,H] (zeros at padding).
-  // sync_count: read the valid-token count back once (exact launch sizes, one stream synchronisation, as the reference
-  // does in every layer) or leave it on the device (no synchronisation, launches sized for B*S rows).
+  // sync_count: read the valid-token count back once per batch, so that the launches of layers 2 .. L are sized
+  // exactly (the reference reads it back in every layer), or leave it on the device (launches sized for B*S rows).
+  // The copy is asynchronous and the host waits for it behind the launches of the first layer, which is sized for
+  // B*S rows and bounded on the device, so the GPU never idles for the read-back.
   // Returns the valid-token count, or -1 when it was not read back.
   int forward(const void* from_tensor, const int32_t* mask, const void* attr_mask, void* out, int batch, int seq_len,
               hipStream_t stream, bool sync_count = true) {
@@ -119,23 +128,39 @@ class Encoder {
     void* ws = ws_.reserve(in_ws > layer_ws ? in_ws : layer_ws);
     int32_t host_count = -1;
     check(et_input(handle_.get(), dtype_, from_tensor, mask, act, count, batch_idx, word_idx, batch, seq_len, heads_, d_, ws,
-                   ws_.capacity(), stream, sync_count ? &host_count : nullptr),
+                   ws_.capacity(), stream, nullptr),
           handle_.get());
+    bool pending = false;
+    if (sync_count) {
+      if (!host_count_) check_hip(hipHostMalloc((void**)&host_count_, sizeof(int32_t), hipHostMallocDefault), "hipHostMalloc");
+      if (!copied_) check_hip(hipEventCreateWithFlags(&copied_, hipEventDisableTiming), "hipEventCreate");
+      check_hip(hipMemcpyAsync(host_count_, count, sizeof(int32_t), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+      check_hip(hipEventRecord(copied_, stream), "hipEventRecord");
+      pending = true;
+    }
     // one sequence start table serves every layer of the batch
     check(et_sequence_starts(handle_.get(), batch_idx, count, batch, seq_len, starts, stream), handle_.get());
     const char* x = act;
     for (size_t l = 0; l < layers_.size(); ++l) {
+      if (l == 1 && pending) {       // the first layer is in the queue: waiting here leaves the GPU with work
+        check_hip(hipEventSynchronize(copied_), "hipEventSynchronize");
+        host_count = *host_count_;
+        pending = false;
+      }
       char* y = act + (1 + (l & 1)) * rows * H * e;
       et_layer_prepared prep = prepared_[l];
       prep.seq_start = starts;
       check(et_layer_with_prepared(handle_.get(), dtype_, &layers_[l], &prep, x, x, attr_mask, count, batch_idx, word_idx, y,
-                                   batch, seq_len, seq_len, heads_, d_, sync_count ? host_count : -1, ws, ws_.capacity(),
-                                   stream),
+                                   batch, seq_len, seq_len, heads_, d_, host_count, ws, ws_.capacity(), stream),
             handle_.get());
       x = y;
     }
     check(et_output(handle_.get(), dtype_, x, count, batch_idx, word_idx, out, batch, seq_len, heads_, d_, stream),
           handle_.get());
+    if (pending) {                   // a single layer: nothing needed the count, the caller still gets it
+      check_hip(hipEventSynchronize(copied_), "hipEventSynchronize");
+      host_count = *host_count_;
+    }
     return host_count;
   }
 
@@ -146,6 +171,8 @@ class Encoder {
   std::vector<et_layer_weights> layers_;
   std::vector<et_layer_prepared> prepared_;
   DeviceBuffer act_, idx_, ws_, wt_;
+  int32_t* host_count_ = nullptr;      // pinned
+  hipEvent_t copied_ = nullptr;
 };
 
 }  // namespace et
