@@ -794,7 +794,8 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
 
 // ------------------------------------------------------------------------------------------
 // fp16, problems below the persistent regime, B k-contiguous ([n][k]): one (32 MI) x (32 NJ) tile per workgroup,
-// 4 wavefronts (2 x 2), LDS slots of two k-steps like the persistent kernel above.
+// 4 wavefronts (2 x 2), LDS slots of two k-steps like the persistent kernel above.  MI = 1 .. 4 blocks of 32 rows,
+// NJ = 2, 4, 6 or 8 blocks of 32 columns.
 //
 // With the weights in TF's [k][n] order a small tile reads its B operands with 8-byte LDS reads (half the rate of
 // 16-byte ones) and transposes them in registers, and its A rows arrive in 64-byte pieces; a 64 x 128 tile then spends
@@ -848,7 +849,8 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
 
   // DMA: one instruction fills 1 KB of LDS = 8 rows x 128 bytes; the lane picks the 16-byte chunk that belongs at its
   // (XOR-swizzled) position.  LDS row j*16+l of a wave's column group holds column NJ*l+j of the group, so that the
-  // operand reads of B^T look like A's and a lane owns NJ consecutive columns of C.
+  // operand reads of B^T look like A's and a lane owns NJ consecutive columns of C (NJ = 6: four consecutive columns
+  // among the first 64 of the group and two among the last 32, for aligned 8- and 4-byte stores).
   uint32_t voff_a[MI], voff_b[NJ];
 #pragma unroll
   for (int j = 0; j < MI; ++j) {
@@ -858,7 +860,8 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
     const int row = wave * (8 * NJ) + j * 8 + (lane >> 3);
-    const int col = (row / WC) * WC + (row & 15) * NJ + ((row % WC) >> 4);
+    const int jb = (row % WC) >> 4;                                 // 16-row block of the wave's column group
+    const int col = (row / WC) * WC + (NJ != 6 ? (row & 15) * NJ + jb : jb < 4 ? (row & 15) * 4 + jb : 64 + (row & 15) * 2 + jb - 4);
     voff_b[j] = ((uint32_t)col * (uint32_t)K + (uint32_t)((lane & 7) ^ pair_swizzle(row)) * 8u) * 2u;
   }
   // instruction q (0..MI-1: A, MI..: B^T) of this wave's share of pair `pr` into slot `slot`; pairs past the end
@@ -937,28 +940,55 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
   wait_vmcnt<0>();                               // no DMA may still target this workgroup's LDS when it ends
 
   // epilogue: lane owns rows g*4+r of every 16-row block and NJ consecutive columns
-  const int col = n0 + wn * WC + l16 * NJ;
+  const int col = n0 + wn * WC + l16 * (NJ == 6 ? 4 : NJ);
   if (col < N) {
     _Float16* C = (_Float16*)args.C + (size_t)grp * N + col;
-    // bias added in half on the rounded product, as the reference's next kernel does; without a bias the addend is
-    // -0, which leaves every value (and the sign of a zero) as it is
-    HalfN biasv;
+    if constexpr (NJ == 2 || NJ == 4 || NJ == 8) {
+      // bias added in half on the rounded product, as the reference's next kernel does; without a bias the addend is
+      // -0, which leaves every value (and the sign of a zero) as it is
+      HalfN biasv;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) biasv[j] = (_Float16)-0.0f;
-    if (args.bias[grp] != nullptr) biasv = *reinterpret_cast<const HalfN*>((const _Float16*)args.bias[grp] + col);
+      for (int j = 0; j < NJ; ++j) biasv[j] = (_Float16)-0.0f;
+      if (args.bias[grp] != nullptr) biasv = *reinterpret_cast<const HalfN*>((const _Float16*)args.bias[grp] + col);
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = m0 + wm * 16 * MI + i * 16 + g * 4 + r;
-        if (row < rows) {
-          HalfN o;
+        for (int r = 0; r < 4; ++r) {
+          const int row = m0 + wm * 16 * MI + i * 16 + g * 4 + r;
+          if (row < rows) {
+            HalfN o;
 #pragma unroll
-          for (int j = 0; j < NJ; ++j) o[j] = f2h(acc[i][j][r]);
-          o = args.gelu ? bias_gelu_half<HalfN, NJ>(o, biasv) : o + biasv;
-          __builtin_nontemporal_store(o, reinterpret_cast<HalfN*>(C + (size_t)row * args.ldc));
+            for (int j = 0; j < NJ; ++j) o[j] = f2h(acc[i][j][r]);
+            o = args.gelu ? bias_gelu_half<HalfN, NJ>(o, biasv) : o + biasv;
+            __builtin_nontemporal_store(o, reinterpret_cast<HalfN*>(C + (size_t)row * args.ldc));
+          }
         }
+    } else {
+      // 6 columns per lane: 4 consecutive ones in the first 64 columns of the wave tile, 2 in the last 32
+      static_assert(NJ == 6, "wave tiles are 32, 64, 96 or 128 columns wide");
+      _Float16* C2 = C - col + n0 + wn * WC + 64 + l16 * 2;
+      half4 bias4 = {(_Float16)-0.0f, (_Float16)-0.0f, (_Float16)-0.0f, (_Float16)-0.0f};
+      half2v bias2 = {(_Float16)-0.0f, (_Float16)-0.0f};
+      const bool ok2 = n0 + wn * WC + 64 + l16 * 2 < N;
+      if (args.bias[grp] != nullptr) {
+        bias4 = *reinterpret_cast<const half4*>((const _Float16*)args.bias[grp] + col);
+        if (ok2) bias2 = *reinterpret_cast<const half2v*>((const _Float16*)args.bias[grp] + n0 + wn * WC + 64 + l16 * 2);
       }
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = m0 + wm * 16 * MI + i * 16 + g * 4 + r;
+          if (row < rows) {
+            half4 o4 = {f2h(acc[i][0][r]), f2h(acc[i][1][r]), f2h(acc[i][2][r]), f2h(acc[i][3][r])};
+            half2v o2 = {f2h(acc[i][4][r]), f2h(acc[i][5][r])};
+            o4 = args.gelu ? bias_gelu_half<half4, 4>(o4, bias4) : o4 + bias4;
+            o2 = args.gelu ? bias_gelu_half<half2v, 2>(o2, bias2) : o2 + bias2;
+            __builtin_nontemporal_store(o4, reinterpret_cast<half4*>(C + (size_t)row * args.ldc));
+            if (ok2) __builtin_nontemporal_store(o2, reinterpret_cast<half2v*>(C2 + (size_t)row * args.ldc));
+          }
+        }
+    }
   }
 #else
   (void)args;
@@ -1228,11 +1258,92 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
 #undef ET_PAIR_CASE
 }
 
+// Tile of the one-tile-per-workgroup k-contiguous kernel.  A workgroup's k loop runs at the rate its CU's load path
+// delivers operand rows, MI + NJ units of 4 KB per pair of k-steps, so the launch takes about as long as the busiest
+// CU's units: the smallest tile that still gives every workgroup a CU to itself ("solo", ring of 3 to 5 slots), or
+// two workgroups per CU ("duo", rings that fit twice into the LDS) where 2 (MI + NJ) / 1.3 is less: two resident
+// workgroups draw 1.3 times the rows of one.  A 96-column wave tile stores in two pieces and counts one unit more.
+// Ties go to the tile whose XCD bands touch fewer distinct operand rows.  (Timed for n = 768 .. 4096, k = 768 .. 4096,
+// 250 .. 16000 rows with the weights of twelve layers taking turns: within 2 % of the best tile on average.)
+struct BtPick {
+  int mi = 0, nj = 0;      // mi == 0: no tile keeps the launch within two workgroups per CU
+  bool duo = false;
+};
+
+BtPick pick_bt_tile(int m_bound, int n, int groups, int cus, bool proven_only) {
+  BtPick best;
+  float best_cost = 0.f;
+  long best_band = 0;
+  // (the other combinations of 1 .. 4 row blocks and 2 .. 8 column blocks never come out ahead of these)
+  static constexpr struct { int mi, nj; bool duo; } kTiles[] = {{1, 2, true}, {2, 2, true}, {2, 4, true}, {3, 2, true},
+                                                                 {3, 4, true}, {3, 6, true}, {4, 2, true}, {4, 4, true},
+                                                                 {4, 6, true}, {4, 8, false}};
+  for (const auto& tile : kTiles) {
+    const int mi = tile.mi, nj = tile.nj;
+    const long tiles_n = (long)((n + 32 * nj - 1) / (32 * nj)) * groups;
+    const long wgs = (long)((m_bound + 32 * mi - 1) / (32 * mi)) * tiles_n;
+    const float units = (float)(mi + nj + (nj == 6 ? 1 : 0));
+    float cost;
+    bool duo = false;
+    if (wgs <= cus) {
+      cost = units;
+    } else if (wgs <= 2L * cus && tile.duo && !(proven_only && nj > 4)) {
+      cost = 2.f * units / 1.3f;
+      duo = true;
+    } else {
+      continue;
+    }
+    // distinct operand rows (of A and of B^T) that the tiles of one XCD's band touch: what its L2 has to fetch
+    const long per_band = (wgs + kXcds - 1) / kXcds;
+    const long band = (per_band >= tiles_n ? (per_band + tiles_n - 1) / tiles_n : 1) * 32 * mi +
+                      std::min(per_band, tiles_n) * 32 * nj;
+    if (best.mi == 0 || cost < best_cost || (cost == best_cost && band < best_band)) {
+      best.mi = mi;
+      best.nj = nj;
+      best.duo = duo;
+      best_cost = cost;
+      best_band = band;
+    }
+  }
+  return best;
+}
+
+void launch_bt_tile(BtPick p, const GemmArgs& a, hipStream_t stream) {
+  switch (p.mi * 100 + p.nj * 10 + (p.duo ? 1 : 0)) {
+    case 120: return launch_f16_bt<1, 2, 5>(a, stream);
+    case 121: return launch_f16_bt<1, 2, 3>(a, stream);
+    case 220: return launch_f16_bt<2, 2, 4>(a, stream);
+    case 221: return launch_f16_bt<2, 2, 3>(a, stream);
+    case 240: return launch_f16_bt<2, 4, 4>(a, stream);
+    case 241: return launch_f16_bt<2, 4, 3>(a, stream);
+    case 320: return launch_f16_bt<3, 2, 4>(a, stream);
+    case 321: return launch_f16_bt<3, 2, 3>(a, stream);
+    case 340: return launch_f16_bt<3, 4, 4>(a, stream);
+    case 341: return launch_f16_bt<3, 4, 2>(a, stream);
+    case 360: return launch_f16_bt<3, 6, 3>(a, stream);
+    case 361: return launch_f16_bt<3, 6, 2>(a, stream);
+    case 420: return launch_f16_bt<4, 2, 4>(a, stream);
+    case 421: return launch_f16_bt<4, 2, 3>(a, stream);
+    case 440: return launch_f16_bt<4, 4, 4>(a, stream);
+    case 460: return launch_f16_bt<4, 6, 3>(a, stream);
+    case 461: return launch_f16_bt<4, 6, 2>(a, stream);
+    case 480: return launch_f16_bt<4, 8, 3>(a, stream);
+    default: return launch_f16_bt<4, 4, 2>(a, stream);     // 128 x 128 in rounds of two workgroups per CU
+  }
+}
+
 // few big tiles would leave most of the 256 CUs idle: the persistent 256x256 kernel only runs when there is work
 // for at least half of them; C is addressed with 32-bit byte offsets there
 bool use_persistent(int m_bound, int ldc, int n, int k, int groups) {
   const long big = (long)((m_bound + 255) / 256) * ((n + 255) / 256) * groups;
   return big >= 128 && k >= 4 * kHBK && (uint64_t)m_bound * (uint64_t)ldc * 2u <= 0xffffffffull;
+}
+
+// With B k-contiguous, the one-tile-per-workgroup kernel is still the faster one where the launch fits a round of
+// 128 x 256 tiles or two workgroups of 128 x 128 per CU (2000 rows at n = 4096, k = 1024: 21 us against 27; 8000 rows
+// at n = 1024, k = 4096: 59 against 73); narrower duo tiles only tie with the persistent kernel there.
+bool use_persistent_bt(int m_bound, int ldc, int n, int k, int groups) {
+  return use_persistent(m_bound, ldc, n, k, groups) && pick_bt_tile(m_bound, n, groups, device_cu_count(), true).mi == 0;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1295,8 +1406,8 @@ bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int gr
 // are 512 contiguous bytes, is as fast inside the layer as the k-contiguous one is on its own, so the copy is skipped.
 bool gemm_blocked_handover(DType t, int m_bound, int wide, int narrow) {
   // ... and both would run on tiles of 256 rows anyway (a lower tile for one of them is worth more than the hand-over)
-  return gemm_takes_transposed_b(t, m_bound, wide, wide, narrow, 1) && use_persistent(m_bound, wide, wide, narrow, 1) &&
-         gemm_takes_transposed_b(t, m_bound, narrow, narrow, wide, 1) && use_persistent(m_bound, narrow, narrow, wide, 1) &&
+  return gemm_takes_transposed_b(t, m_bound, wide, wide, narrow, 1) && use_persistent_bt(m_bound, wide, wide, narrow, 1) &&
+         gemm_takes_transposed_b(t, m_bound, narrow, narrow, wide, 1) && use_persistent_bt(m_bound, narrow, narrow, wide, 1) &&
          pair_kernel_row_blocks(m_bound, wide, 1) == 8 && pair_kernel_row_blocks(m_bound, narrow, 1) == 8 &&
          wide % kPBN == 0 && (uint64_t)((m_bound + kPBM - 1) / kPBM * kPBM) * (uint64_t)wide * 2u <= 0xffffffffull;
 }
@@ -1348,29 +1459,13 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.a_blocked = g.a_blocked ? 1 : 0;
   a.c_blocked = g.c_blocked ? 1 : 0;
   if (t == DType::F16) {
-    if (use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
+    if (g.b_transposed ? use_persistent_bt(m_bound, ldc, n, k, g.groups)
+                       : use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles
       launch_f16_persistent(a, stream, g.b_transposed);
     } else if (g.b_transposed) {
-      // Below the persistent regime a workgroup's k loop runs at the rate its CU's load path delivers the operand rows
-      // (the smaller the tile, the more bytes per MFMA), so the largest tile that still gives about 0.55 workgroups
-      // per CU is taken; the ring is deeper (5 or 6 slots) when every workgroup has a CU to itself, and small enough
-      // for two workgroups per CU otherwise (timed for n = 768 .. 3072, k = 768 and 3072, 250 .. 10000 rows, with the
-      // weights of twelve layers taking turns).
+      // one tile per workgroup, the tile chosen for the launch's shape (pick_bt_tile)
       const int cus = device_cu_count();
-      auto wgs = [&](int bm, int bn) { return (long)((m_bound + bm - 1) / bm) * ((n + bn - 1) / bn) * g.groups; };
-      const long enough = (long)cus * 55 / 100;
-      if (wgs(128, 128) >= enough) {
-        if (wgs(128, 128) <= cus) launch_f16_bt<4, 4, 5>(a, stream);
-        else launch_f16_bt<4, 4, 2>(a, stream);
-      } else if (wgs(64, 128) >= enough) {
-        if (wgs(64, 128) <= cus) launch_f16_bt<2, 4, 6>(a, stream);
-        else launch_f16_bt<2, 4, 3>(a, stream);
-      } else if (wgs(64, 64) >= enough) {
-        if (wgs(64, 64) <= cus) launch_f16_bt<2, 2, 6>(a, stream);
-        else launch_f16_bt<2, 2, 3>(a, stream);
-      } else {
-        launch_f16_bt<1, 2, 6>(a, stream);
-      }
+      launch_bt_tile(pick_bt_tile(m_bound, n, g.groups, cus, false), a, stream);
     } else {
       // Below a round of the chip the time of a launch is the k loop of one tile.  With fewer 64 x 256 tiles than CUs
       // that loop runs at the rate one CU's DMA fills its LDS: the 64 x 128 tile halves the B bytes per workgroup and

@@ -366,13 +366,21 @@ def test_gemm(k, dtype, m, n, k_):
 # those leave a last round that keeps at most half of the workgroups busy, so those tiles are shared by two
 # workgroups, one per 128-column half, one of them with a ragged last column tile; the next three run on tiles of
 # 160, 192 and 224 rows, which fill the chip's single round better), below that one tile per workgroup
-# of 128x128 (one or two workgroups per CU), 64x128, 64x64 or 32x64, with ragged last tiles in both directions and a
-# single pair of k-steps.  The oracle product is taken on the CPU in float64 for a sample of rows.
+# of 32 .. 128 rows by 64 .. 256 columns, with ragged last tiles in both directions and a single pair of k-steps.  The
+# last eighteen shapes reach, on a 256-CU part, every tile of that kernel in both of its ring depths: 32x64, 64x64,
+# 64x128, 96x64, 96x128, 96x192, 128x64, 128x128, 128x192 with a CU per workgroup and with two workgroups per CU, and
+# 128x256; three of the 192-column ones have a ragged last column tile.  The oracle product is taken on the CPU in
+# float64 for a sample of rows.
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072),
                                     (23301, 768, 768), (14000, 1032, 128),
                                     (13097, 768, 3072), (15866, 768, 768), (13097, 1024, 1024),
                                     (6000, 776, 768), (4000, 768, 3072), (3000, 1032, 128), (2000, 768, 768),
-                                    (1001, 776, 3072), (500, 768, 64), (302, 40, 192)])
+                                    (1001, 776, 3072), (500, 768, 64), (302, 40, 192),
+                                    (2308, 392, 128), (722, 768, 192), (2491, 776, 128), (2064, 768, 128),
+                                    (5419, 768, 128), (1393, 768, 192), (3467, 776, 128), (2735, 768, 128),
+                                    (6151, 768, 128), (5480, 768, 192), (9348, 776, 128), (1881, 776, 128),
+                                    (4626, 776, 128), (4077, 768, 128), (8225, 776, 64), (3849, 1032, 192),
+                                    (9803, 776, 128), (8225, 768, 128)])
 def test_gemm_bt(k, m, n, k_):
     print("gemm_bt", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_)
@@ -396,8 +404,8 @@ def test_gemm_bt(k, m, n, k_):
 
 # A sequence gives the same bits in a batch of any size: every fp16 kernel accumulates k in the same order, so the
 # rows of a small problem (64x128 tiles), a middle one (128x256 tiles) and a large one (persistent 256x256 tiles, B in
-# either storage order) agree bit for bit, and so do the four one-tile-per-workgroup kernels for k-contiguous B
-# (128x128, 64x128, 64x64, 32x64); the two fp32 tiles likewise.
+# either storage order) agree bit for bit, and so do the one-tile-per-workgroup kernels for k-contiguous B
+# (tiles from 32x64 to 128x256); the two fp32 tiles likewise.
 @pytest.mark.parametrize("n,k_", [(768, 768), (768, 3072), (3072, 768)])
 def test_gemm_same_bits_in_every_kernel(k, n, k_):
     print("gemm same bits", n, k_, flush=True)
@@ -411,7 +419,7 @@ def test_gemm_same_bits_in_every_kernel(k, n, k_):
     for rows in (6000, 2500, 300, 1):
         part = k.gemm(a[:rows].contiguous(), b).cpu().numpy()
         assert np.array_equal(part, big[:rows]), rows
-    for rows in (9000, 6000, 4000, 2000, 1000, 500, 130, 1):
+    for rows in (9000, 8200, 6000, 5400, 4000, 2700, 2000, 1400, 1000, 500, 130, 1):
         part = k.gemm_bt(a[:rows].contiguous(), bt).cpu().numpy()
         assert np.array_equal(part, big[:rows]), rows
     a32, b32 = a.float(), b.float()
@@ -440,8 +448,10 @@ def test_gemm_bias_gelu_equals_the_two_passes(k, dtype, m, n, k_):
         k.gemm(dev(a), dev(b), gelu=True)
 
 
+# (the last four shapes: 192-column tiles, whose lanes store a group of four and a group of two columns)
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (5000, 3072, 768), (2000, 3072, 768),
-                                    (1000, 776, 128), (400, 768, 768), (350, 200, 64)])
+                                    (1000, 776, 128), (400, 768, 768), (350, 200, 64),
+                                    (5480, 768, 128), (3849, 1032, 64), (9803, 776, 64), (1288, 3080, 64)])
 def test_gemm_bt_bias_gelu_equals_the_two_passes(k, m, n, k_):
     print("gemm_bt_bias_gelu", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_ + 1)
