@@ -939,7 +939,9 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
   }
   wait_vmcnt<0>();                               // no DMA may still target this workgroup's LDS when it ends
 
-  // epilogue: lane owns rows g*4+r of every 16-row block and NJ consecutive columns
+  // epilogue: lane owns rows g*4+r of every 16-row block and NJ consecutive columns.  Plain stores, not the
+  // non-temporal ones of the persistent kernel: the output of a launch this small is still in the caches when the
+  // next kernel reads it (12 layers on 2000 tokens: 0.905 -> 0.843 ms; no difference from about 4000 tokens on).
   const int col = n0 + wn * WC + l16 * (NJ == 6 ? 4 : NJ);
   if (col < N) {
     _Float16* C = (_Float16*)args.C + (size_t)grp * N + col;
@@ -960,7 +962,7 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
 #pragma unroll
             for (int j = 0; j < NJ; ++j) o[j] = f2h(acc[i][j][r]);
             o = args.gelu ? bias_gelu_half<HalfN, NJ>(o, biasv) : o + biasv;
-            __builtin_nontemporal_store(o, reinterpret_cast<HalfN*>(C + (size_t)row * args.ldc));
+            *reinterpret_cast<HalfN*>(C + (size_t)row * args.ldc) = o;
           }
         }
     } else {
@@ -984,8 +986,8 @@ __global__ __launch_bounds__(kHThreads) __attribute__((amdgpu_waves_per_eu(2))) 
             half2v o2 = {f2h(acc[i][4][r]), f2h(acc[i][5][r])};
             o4 = args.gelu ? bias_gelu_half<half4, 4>(o4, bias4) : o4 + bias4;
             o2 = args.gelu ? bias_gelu_half<half2v, 2>(o2, bias2) : o2 + bias2;
-            __builtin_nontemporal_store(o4, reinterpret_cast<half4*>(C + (size_t)row * args.ldc));
-            if (ok2) __builtin_nontemporal_store(o2, reinterpret_cast<half2v*>(C2 + (size_t)row * args.ldc));
+            *reinterpret_cast<half4*>(C + (size_t)row * args.ldc) = o4;
+            if (ok2) *reinterpret_cast<half2v*>(C2 + (size_t)row * args.ldc) = o2;
           }
         }
     }
