@@ -53,6 +53,12 @@ namespace {
 // kStaticMaxPositions positions.  Every GPU the library runs on holds its own copy of the array until the process
 // ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use is looked
 // up once per device (et_create) and kept in static_scratch_ptr.
+// The persistent GEMM stores C with plain stores while the matrices of a layer (resp. A and C of a stand-alone call)
+// are small enough to be found in the 256 MB last-level cache by the kernels that read them next, and with non-temporal
+// stores beyond.  12-layer BERT-base, fp16: plain stores -6 % at 4000 tokens, -2.4 % at 15900, +-0.5 % at 20000,
+// +2 % at 30000 and 40000; 24-layer BERT-large at 13100 tokens: -0.4 %.
+constexpr double kCachedLayerBytes = 320.0 * 1048576.0;
+constexpr double kCachedCallBytes = 128.0 * 1048576.0;
 constexpr int kStaticScratchWords = 1024;
 constexpr int kStaticMaxPositions = 1024 * 1024;
 static __device__ __align__(256) int32_t scratch[kStaticScratchWords];
@@ -465,9 +471,14 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
     if (pp.seq_start) seq_start = const_cast<int32_t*>(pp.seq_start);
     et::launch_transpose_weights(jobs, st, pp.seq_start ? nullptr : &seq);
   }
+  // Every matrix of the layer is read again by the kernel after the one that wrote it.  While the layer's matrices
+  // (from, Q/K/V, context, attention output, [T,4H], out) about fit the last-level cache, the GEMMs leave their
+  // outputs there (plain stores); beyond that the outputs would only displace the weights and the A rows.
+  const bool cached = (double)rows * (7.0 * H + F) * (double)e <= kCachedLayerBytes;
   // Q = from.Wq + bq, K = to.Wk + bk, V = to.Wv + bv into one [T,3H] buffer (bert_transformer_op.cu.cc:105-156)
   et::GemmGroups g3;
   g3.groups = 3;
+  g3.c_cached = cached;
   g3.A[0] = from_tensor; g3.A[1] = to_tensor; g3.A[2] = to_tensor;
   g3.B[0] = t_qkv ? wt_q : w->attr_kernel_Q; g3.B[1] = t_qkv ? wt_k : w->attr_kernel_K; g3.B[2] = t_qkv ? wt_v : w->attr_kernel_V;
   g3.bias[0] = w->attr_bias_Q; g3.bias[1] = w->attr_bias_K; g3.bias[2] = w->attr_bias_V;
@@ -481,6 +492,7 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   // attention output projection + bias + residual(from_tensor) + LayerNorm (:195-213)
   et::GemmGroups g1;
   g1.groups = 1;
+  g1.c_cached = cached;
   g1.A[0] = ctx; g1.B[0] = t_o ? wt_o : w->attr_output_kernel; g1.bias[0] = nullptr;
   g1.b_transposed = t_o;
   et::launch_gemm(dt, g1, attn, H, rows, H, H, T, st);
@@ -784,6 +796,7 @@ et_status gemm_bt_impl(et_handle h, et_dtype dtype, const void* A, const void* B
   g.A[0] = A; g.B[0] = Bt; g.bias[0] = bias;
   g.b_transposed = true;
   g.gelu = gelu;
+  g.c_cached = (double)m * ((double)k + n) * 2.0 <= kCachedCallBytes;     // A and C together: a small call
   et::launch_gemm(et::DType::F16, g, C, n, m, n, k, m_dev, (hipStream_t)stream);
   return check_launch(h, what);
 }

@@ -39,6 +39,7 @@ struct GemmArgs {
   int gelu = 0;              // C = gelu(A.B + bias) instead of A.B + bias (bias must be set)
   int a_blocked = 0;         // pair kernel: A / C hold every tile of 256 rows as blocks of [256 rows][64 columns]
   int c_blocked = 0;         //   (see GemmGroups)
+  int c_cached = 0;          // persistent k-contiguous kernel: plain stores for C instead of non-temporal ones
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -546,7 +547,9 @@ __device__ __forceinline__ int pair_swizzle(int row) { return (row >> 1) & 7; }
 // fills whole rounds of the chip; a lower tile can turn "one round and a bit" into one round (launch_f16_persistent
 // chooses).  The A part of an LDS slot keeps its 256 rows; the rows beyond the tile lie outside the tile's buffer
 // descriptor and cost no traffic.
-template <bool GELU, int MI>
+// NT: C leaves through non-temporal stores (a matrix too big to be found in the last-level cache by its reader);
+// plain stores otherwise.
+template <bool GELU, int MI, bool NT>
 __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -774,7 +777,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
             for (int j = 0; j < 4; ++j) o[j] = f2h(acc[i][j][r]);
             // GELU here costs no pass over C: its arithmetic runs while the stores of the tile drain
             o = GELU ? bias_gelu_half<half4, 4>(o, bias4) : o + bias4;
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, o), rc, voff, 0, 2 /* nt */);
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2v, o), rc, voff, 0, NT ? 2 /* nt */ : 0);
             voff += row_bytes;
           }
           voff += 12u * row_bytes;
@@ -1221,9 +1224,9 @@ int pair_kernel_row_blocks(int m_bound, int n, int groups) {
   return best_mi;
 }
 
-template <bool GELU, int MI>
+template <bool GELU, int MI, bool NT>
 void launch_pair(const GemmArgs& a, int grid, hipStream_t stream) {
-  auto kern = gemm_f16_pair_kernel<GELU, MI>;
+  auto kern = gemm_f16_pair_kernel<GELU, MI, NT>;
   allow_dynamic_lds(reinterpret_cast<const void*>(kern), kQSmem);
   kern<<<grid, kPThreads, kQSmem, stream>>>(a);
 }
@@ -1246,10 +1249,12 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
     gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
     return;
   }
-#define ET_PAIR_CASE(M)                                  \
-  case M:                                                \
-    if (a.gelu) launch_pair<true, M>(a, grid, stream);   \
-    else launch_pair<false, M>(a, grid, stream);         \
+#define ET_PAIR_CASE(M)                                                      \
+  case M:                                                                    \
+    if (a.gelu && a.c_cached) launch_pair<true, M, false>(a, grid, stream);  \
+    else if (a.gelu) launch_pair<true, M, true>(a, grid, stream);            \
+    else if (a.c_cached) launch_pair<false, M, false>(a, grid, stream);      \
+    else launch_pair<false, M, true>(a, grid, stream);                       \
     break;
   switch (mi) {
     ET_PAIR_CASE(8)
@@ -1460,6 +1465,7 @@ void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, in
   a.gelu = g.gelu ? 1 : 0;
   a.a_blocked = g.a_blocked ? 1 : 0;
   a.c_blocked = g.c_blocked ? 1 : 0;
+  a.c_cached = g.c_cached ? 1 : 0;
   if (t == DType::F16) {
     if (g.b_transposed ? use_persistent_bt(m_bound, ldc, n, k, g.groups)
                        : use_persistent(m_bound, ldc, n, k, g.groups)) {     // one workgroup per CU walks the tiles

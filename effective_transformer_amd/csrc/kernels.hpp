@@ -102,6 +102,10 @@ struct GemmGroups {
   // and pair of k-steps, are contiguous in memory instead of one row stride apart.  Only where
   // gemm_blocked_handover() says so; the matrix must be allocated for a whole number of 256-row tiles.
   bool c_blocked = false, a_blocked = false;
+  // C is read again by the next kernels while it can still be in the last-level cache (the working set of the layer
+  // or of the call fits it a few times over): the persistent kernel then stores C with plain stores.  Its non-temporal
+  // stores are the better choice when C would only push the weights and the A rows out of that cache.
+  bool c_cached = false;
 };
 bool gemm_supported(DType t, int n, int k, int groups);
 // True when both C = A.B1 ([m, wide] from k = narrow) and the product that consumes it (k = wide, n = narrow) run the
