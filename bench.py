@@ -25,7 +25,7 @@ if ROOT not in sys.path:
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # kernel name in the counter files -> key in `kernels`, for the kernels one name identifies (the FFN-up projection is the
 # only launch of the GELU instance of the large-M GEMM; the other three projections share one instance)
-TRAFFIC_KERNELS = (("gemm_f16_pair_kernel<true>", "gemm_ffn_up"), ("gemm_f16_pair_kernelILb1", "gemm_ffn_up"),
+TRAFFIC_KERNELS = (("gemm_f16_pair_kernel<true,", "gemm_ffn_up"), ("gemm_f16_pair_kernelILb1", "gemm_ffn_up"),
                    ("attention_kernel", "attention"), ("attention_long_kernel", "attention"),
                    ("bias_residual_layernorm_kernel", "bias_residual_layernorm"), ("bias_gelu_kernel", "bias_gelu"),
                    ("restore_rows_kernel", "output_restore"))
