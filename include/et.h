@@ -114,9 +114,11 @@ et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, 
  * (op registered at tf_op/bert_transformer_op.cc:44-77): one encoder layer on packed tokens.
  *   from_tensor, to_tensor [T,H] packed; attr_mask [B,S,S] of dtype (1 = attend);
  *   out [T,H] packed (rows >= T untouched).
- * valid_word_num_hint: T when the host knows it (grids are sized exactly), or -1: grids are
- * then sized for B*S rows and every kernel bounds itself by *valid_word_num_dev, so the call
- * never blocks the host (the reference copies T back every layer, :99-101).
+ * valid_word_num_hint: T when the host knows it (grids are sized exactly), any upper bound of T
+ * that the caller vouches for (grids are sized for that many rows; rows beyond it would not be
+ * computed), or -1: grids are then sized for B*S rows.  Every kernel bounds itself by
+ * *valid_word_num_dev, so the call never blocks the host (the reference copies T back every
+ * layer, :99-101).
  * from_seq_len must equal to_seq_len (tf_op/bert_transformer_op.cc:130-131).  `out` must not
  * alias from_tensor/to_tensor.  Shapes: seq_len <= 1024, batch_size <= 65535, size_per_head <= 256 (see et_attention),
  * hidden size a multiple of 32 (fp16) or 16 (fp32). */

@@ -240,6 +240,49 @@ def test_hip_graph_replays_match_eager():
     print("graph/new mask max abs diff", _check(got2.cpu().numpy(), _oracle(w2), mask2, "fp16"), flush=True)
 
 
+def test_hip_graph_sized_for_a_token_bound():
+    """A graph captured with max_valid_tokens sizes its launches for that many rows instead of B*S: replays with the
+    capture mask, with a shorter one and with one that reaches the bound exactly equal the eager runs bit for bit, and a
+    mask beyond the bound is refused."""
+    from effective_transformer_amd import ops
+    w = o.make_workload("cfg2", layers=2)
+    wl = w["wl"]
+    dt = TDT[wl.dtype]
+    enc = ops.EffectiveTransformerEncoder(2, wl.heads, wl.d, w["weights"], dt, "cuda")
+    x = dev(w["x"], dt); mask = dev(w["mask"]); attr = dev(w["attr_mask"], dt)
+    tokens = int(w["mask"].sum())
+    bound = tokens + 37
+    assert bound < wl.B * wl.S
+    g = enc.make_graph(x, mask, attr, max_valid_tokens=bound)
+    assert torch.equal(g().clone(), enc(x, mask, attr))
+    rng = np.random.RandomState(5)
+    for case in ("shorter", "at the bound"):
+        lens = w["mask"].sum(axis=1)
+        if case == "shorter":
+            lens = np.maximum(lens - rng.randint(0, 8, size=wl.B), 0)
+        else:
+            room = wl.S - lens
+            add = np.zeros_like(lens)
+            left = 37
+            for b in range(wl.B):
+                add[b] = min(room[b], left)
+                left -= add[b]
+            assert left == 0
+            lens = lens + add
+        mask2 = (np.arange(wl.S)[None, :] < lens[:, None]).astype(np.int32)
+        assert mask2.sum() <= bound and (case == "shorter" or mask2.sum() == bound)
+        attr2 = np.ascontiguousarray(np.broadcast_to(mask2[:, None, :], (wl.B, wl.S, wl.S))).astype(np.float16)
+        want = enc(x, dev(mask2), dev(attr2)).clone()
+        got = g(None, dev(mask2), dev(attr2)).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), case
+    full = dev(np.ones((wl.B, wl.S), np.int32))
+    with pytest.raises(ValueError, match="max_valid_tokens"):
+        g(None, full, None)
+    with pytest.raises(ValueError, match="max_valid_tokens"):
+        enc.make_graph(x, full, attr, max_valid_tokens=bound)
+
+
 def test_error_paths():
     from effective_transformer_amd import _lib, ops
     lib = _lib.load()
