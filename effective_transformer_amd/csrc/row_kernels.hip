@@ -88,13 +88,24 @@ template <int VEC> struct RowVec<_Float16, VEC> {
 template <typename T, int VEC, int ITERS>
 __global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
     T* __restrict__ out, const T* __restrict__ input, const T* __restrict__ bias, const T* __restrict__ gamma,
-    const T* __restrict__ beta, int m, int n, const int32_t* __restrict__ rows_dev) {
+    const T* __restrict__ beta, int m, int n, const int32_t* __restrict__ rows_dev,
+    const uint32_t* __restrict__ warm, int warm_lines) {
   using V = typename RowVec<T, VEC>::type;
   const int rows = rows_dev ? min(*rows_dev, m) : m;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = blockIdx.x * kLnWaves + threadIdx.x / kWave;
   const int nwaves = gridDim.x * kLnWaves;
   const int vpr = n / VEC;                       // vectors per row
+
+  // `warm`: a region (a weight matrix) that the kernel after the next one reads cold; one word of each of its 128-byte
+  // lines is requested here, which pulls the line into the last-level cache.  The values are only looked at behind
+  // the row loop, so no wavefront waits for them.
+  uint32_t warm0 = 0, warm1 = 0;
+  if (warm != nullptr) {
+    const int tid = blockIdx.x * kLnThreads + threadIdx.x, nth = gridDim.x * kLnThreads;
+    if (tid < warm_lines) warm0 = warm[(size_t)tid * 32];
+    for (int i = tid + nth; i < warm_lines; i += nth) warm1 ^= warm[(size_t)i * 32];
+  }
 
   V b[ITERS], g[ITERS], be[ITERS];
 #pragma unroll
@@ -156,6 +167,8 @@ __global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
       }
     }
   }
+  // never true (rows >= 0); keeps the requests above alive
+  if (rows < 0 && (warm0 ^ warm1) == 0x9e3779b9u) out[0] = (T)0;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -262,11 +275,11 @@ bool ln_pick(int n, int& vec, int& iters) {
 
 template <typename T, int VEC>
 void ln_launch_iters(int iters, int grid, hipStream_t stream, T* out, const T* input, const T* bias, const T* gamma,
-                     const T* beta, int m, int n, const int32_t* rows_dev) {
+                     const T* beta, int m, int n, const int32_t* rows_dev, const uint32_t* warm, int warm_lines) {
 #define ET_LN_CASE(I)                                                                                          \
   case I:                                                                                                      \
     bias_residual_layernorm_kernel<T, VEC, I><<<grid, kLnThreads, 0, stream>>>(out, input, bias, gamma, beta, m, n, \
-                                                                               rows_dev);                      \
+                                                                               rows_dev, warm, warm_lines);    \
     break;
   switch (iters) {
     ET_LN_CASE(1)
@@ -283,7 +296,9 @@ void ln_launch_iters(int iters, int grid, hipStream_t stream, T* out, const T* i
 
 template <typename T>
 void ln_launch(void* out, const void* input, const void* bias, const void* gamma, const void* beta, int m, int n,
-               const int32_t* rows_dev, hipStream_t stream) {
+               const int32_t* rows_dev, hipStream_t stream, const void* warm_region, size_t warm_bytes) {
+  const uint32_t* warm = (const uint32_t*)warm_region;
+  const int warm_lines = warm ? (int)std::min<size_t>(warm_bytes / 128, 1u << 24) : 0;
   int vec = 0, iters = 0;
   if (!ln_pick<T>(n, vec, iters)) return;
   // enough wavefronts to fill 256 CUs several times over; rows beyond that are looped
@@ -292,11 +307,11 @@ void ln_launch(void* out, const void* input, const void* bias, const void* gamma
   const T *i = (const T*)input, *b = (const T*)bias, *g = (const T*)gamma, *be = (const T*)beta;
   constexpr int MV = 16 / (int)sizeof(T);
   if (vec == MV)
-    ln_launch_iters<T, MV>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
+    ln_launch_iters<T, MV>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm, warm_lines);
   else if (vec == MV / 2)
-    ln_launch_iters<T, MV / 2>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
+    ln_launch_iters<T, MV / 2>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm, warm_lines);
   else
-    ln_launch_iters<T, MV / 4>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev);
+    ln_launch_iters<T, MV / 4>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm, warm_lines);
 }
 
 struct EmbedArgs {
@@ -377,11 +392,12 @@ bool bias_residual_layernorm_supported(DType t, int n) {
 }
 
 void launch_bias_residual_layernorm(DType t, void* out, const void* input, const void* bias, const void* gamma,
-                                    const void* beta, int m, int n, const int32_t* rows_dev, hipStream_t stream) {
+                                    const void* beta, int m, int n, const int32_t* rows_dev, hipStream_t stream,
+                                    const void* warm_region, size_t warm_bytes) {
   if (t == DType::F32)
-    ln_launch<float>(out, input, bias, gamma, beta, m, n, rows_dev, stream);
+    ln_launch<float>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm_region, warm_bytes);
   else
-    ln_launch<_Float16>(out, input, bias, gamma, beta, m, n, rows_dev, stream);
+    ln_launch<_Float16>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm_region, warm_bytes);
 }
 
 }  // namespace et
