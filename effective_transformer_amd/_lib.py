@@ -31,7 +31,7 @@ class LayerWeights(C.Structure):
 class LayerPrepared(C.Structure):
     _fields_ = [("attr_kernel_Q_t", C.c_void_p), ("attr_kernel_K_t", C.c_void_p), ("attr_kernel_V_t", C.c_void_p),
                 ("attr_output_kernel_t", C.c_void_p), ("inter_kernel_t", C.c_void_p), ("output_kernel_t", C.c_void_p),
-                ("seq_start", C.c_void_p)]
+                ("seq_start", C.c_void_p), ("warm", C.c_void_p), ("warm_bytes", C.c_size_t)]
 
 
 class EmbeddingWeights(C.Structure):

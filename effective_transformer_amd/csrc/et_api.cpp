@@ -435,7 +435,7 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   // The large-M fp16 GEMM reads k-contiguous weights with fewer LDS instructions.  Where the caller prepared such
   // copies they are used wherever that kernel runs; otherwise the wide projections get a transposed copy in the
   // workspace on every call (the caller's weights stay as they are).
-  static const et_layer_prepared kNoPrep = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  static const et_layer_prepared kNoPrep = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
   const et_layer_prepared& pp = prep ? *prep : kNoPrep;
   ET_REQUIRE(h, (pp.attr_kernel_Q_t != nullptr) == (pp.attr_kernel_K_t != nullptr) &&
                     (pp.attr_kernel_Q_t != nullptr) == (pp.attr_kernel_V_t != nullptr),
@@ -497,16 +497,20 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   g1.A[0] = ctx; g1.B[0] = t_o ? wt_o : w->attr_output_kernel; g1.bias[0] = nullptr;
   g1.b_transposed = t_o;
   et::launch_gemm(dt, g1, attn, H, rows, H, H, T, st);
-  // FFN-down at these sizes is a single round of tiles whose k loop waits for every slice of a weight matrix that was
-  // last read a whole batch ago (13000 rows: 63 us with the weights cold, 53 with them in the last-level cache).  The
-  // LayerNorm in front of FFN-up requests the matrix on its way, while the layer's matrices are small enough for it to
-  // survive FFN-up (12-layer BERT-base: -3 % at 4000 tokens, -4.4 % at 8000 and 12000, -1 % at 16000, nothing beyond)
-  // and the matrix is small beside what the LayerNorm moves anyway.
-  const bool warm_down = t_down && rows >= F && (double)rows * (7.0 * H + F) * (double)e <= kWarmLayerBytes &&
-                         ((uintptr_t)wt_down & 127) == 0;
+  // Every weight matrix was last read a whole batch ago, and a GEMM's first round of tiles waits for each cold slice of
+  // it (13000 rows: FFN-down 63 us with cold weights, 53 with the weights in the last-level cache; 2 .. 3 us for the
+  // other projections).  The two LayerNorm kernels request the matrices that come next on their way, for batches in
+  // which those are small beside what the kernel moves anyway: this one the FFN-up weights and, while the layer's
+  // matrices are small enough for them to survive FFN-up, the FFN-down weights (12-layer BERT-base: -3 % at 4000
+  // tokens, -4.4 % at 8000 and 12000, -1 % at 16000); the last one the region the caller names, the next layer's
+  // attention weights (another -0.7 .. -1.6 % from 4000 to 40000 tokens, FFN-up included).
+  const bool warm_fits = (double)rows * (7.0 * H + F) * (double)e <= kWarmLayerBytes;
+  et::WarmList warm1, warm2;
+  if (t_up && rows >= F) warm1.add(wt_up, (size_t)H * F * e);
+  if (t_down && rows >= F && warm_fits) warm1.add(wt_down, (size_t)H * F * e);
+  if (rows >= F) warm2.add(pp.warm, pp.warm_bytes);
   et::launch_bias_residual_layernorm(dt, attn, from_tensor, w->attr_output_bias, w->attr_output_layernorm_gamma,
-                                     w->attr_output_layernorm_beta, rows, H, T, st, warm_down ? wt_down : nullptr,
-                                     (size_t)H * F * e);
+                                     w->attr_output_layernorm_beta, rows, H, T, st, warm1);
   if ((s = check_launch(h, "attention output")) != ET_OK) return s;
   // FFN up + bias + GELU (:215-227, cuda/cuda_kernels.cu:88-150)
   g1.A[0] = attn; g1.B[0] = t_up ? wt_up : w->inter_kernel;
@@ -526,7 +530,7 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   et::launch_gemm(dt, g1, out, H, rows, H, F, T, st);
   g1.a_blocked = false;
   et::launch_bias_residual_layernorm(dt, out, attn, w->output_bias, w->output_layernorm_gamma,
-                                     w->output_layernorm_beta, rows, H, T, st);
+                                     w->output_layernorm_beta, rows, H, T, st, warm2);
   if ((s = check_launch(h, "FFN down")) != ET_OK) return s;
   return ET_OK;
 }

@@ -53,12 +53,18 @@ bool bias_gelu_supported(DType t, int n);
 void launch_bias_gelu(DType t, void* out, const void* bias, int m, int n, const int32_t* rows_dev,
                       hipStream_t stream);
 bool bias_residual_layernorm_supported(DType t, int n);
-// warm_region: optional, 128-byte aligned; its lines are requested on the way (pulled into the last-level cache) for a
-// later kernel that would otherwise read them cold.
+// Regions whose 128-byte lines a kernel requests on its way (pulled into the last-level cache) for a later kernel that
+// would otherwise read them cold.
+struct WarmList {
+  static constexpr int kMax = 3;
+  const uint32_t* p[kMax] = {nullptr, nullptr, nullptr};
+  int lines[kMax] = {0, 0, 0};
+  int total = 0;
+  void add(const void* region, size_t bytes);
+};
 void launch_bias_residual_layernorm(DType t, void* out, const void* input, const void* bias,
                                     const void* gamma, const void* beta, int m, int n,
-                                    const int32_t* rows_dev, hipStream_t stream,
-                                    const void* warm_region = nullptr, size_t warm_bytes = 0);
+                                    const int32_t* rows_dev, hipStream_t stream, const WarmList& warm = WarmList());
 
 // out[t,:] = LayerNorm(word[ids[p]] + type[type_ids[p]] + pos[word_idx[t]]) * gamma + beta for packed row t at padded
 // position p = batch_idx[t]*seq_len + word_idx[t]; eps 1e-12.  type_ids/type_table and pos_table may be null.

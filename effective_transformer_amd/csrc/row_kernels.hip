@@ -88,8 +88,7 @@ template <int VEC> struct RowVec<_Float16, VEC> {
 template <typename T, int VEC, int ITERS>
 __global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
     T* __restrict__ out, const T* __restrict__ input, const T* __restrict__ bias, const T* __restrict__ gamma,
-    const T* __restrict__ beta, int m, int n, const int32_t* __restrict__ rows_dev,
-    const uint32_t* __restrict__ warm, int warm_lines) {
+    const T* __restrict__ beta, int m, int n, const int32_t* __restrict__ rows_dev, WarmList warm) {
   using V = typename RowVec<T, VEC>::type;
   const int rows = rows_dev ? min(*rows_dev, m) : m;
   const int lane = threadIdx.x & (kWave - 1);
@@ -97,14 +96,19 @@ __global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
   const int nwaves = gridDim.x * kLnWaves;
   const int vpr = n / VEC;                       // vectors per row
 
-  // `warm`: a region (a weight matrix) that the kernel after the next one reads cold; one word of each of its 128-byte
+  // `warm`: regions (weight matrices) that one of the next kernels would read cold; one word of each of their 128-byte
   // lines is requested here, which pulls the line into the last-level cache.  The values are only looked at behind
   // the row loop, so no wavefront waits for them.
   uint32_t warm0 = 0, warm1 = 0;
-  if (warm != nullptr) {
+  if (warm.total > 0) {
     const int tid = blockIdx.x * kLnThreads + threadIdx.x, nth = gridDim.x * kLnThreads;
-    if (tid < warm_lines) warm0 = warm[(size_t)tid * 32];
-    for (int i = tid + nth; i < warm_lines; i += nth) warm1 ^= warm[(size_t)i * 32];
+    auto word = [&](int i) {
+      int r = 0;
+      while (r + 1 < WarmList::kMax && i >= warm.lines[r]) i -= warm.lines[r++];
+      return warm.p[r][(size_t)i * 32];
+    };
+    if (tid < warm.total) warm0 = word(tid);
+    for (int i = tid + nth; i < warm.total; i += nth) warm1 ^= word(i);
   }
 
   V b[ITERS], g[ITERS], be[ITERS];
@@ -275,11 +279,11 @@ bool ln_pick(int n, int& vec, int& iters) {
 
 template <typename T, int VEC>
 void ln_launch_iters(int iters, int grid, hipStream_t stream, T* out, const T* input, const T* bias, const T* gamma,
-                     const T* beta, int m, int n, const int32_t* rows_dev, const uint32_t* warm, int warm_lines) {
+                     const T* beta, int m, int n, const int32_t* rows_dev, const WarmList& warm) {
 #define ET_LN_CASE(I)                                                                                          \
   case I:                                                                                                      \
     bias_residual_layernorm_kernel<T, VEC, I><<<grid, kLnThreads, 0, stream>>>(out, input, bias, gamma, beta, m, n, \
-                                                                               rows_dev, warm, warm_lines);    \
+                                                                               rows_dev, warm);                \
     break;
   switch (iters) {
     ET_LN_CASE(1)
@@ -296,9 +300,7 @@ void ln_launch_iters(int iters, int grid, hipStream_t stream, T* out, const T* i
 
 template <typename T>
 void ln_launch(void* out, const void* input, const void* bias, const void* gamma, const void* beta, int m, int n,
-               const int32_t* rows_dev, hipStream_t stream, const void* warm_region, size_t warm_bytes) {
-  const uint32_t* warm = (const uint32_t*)warm_region;
-  const int warm_lines = warm ? (int)std::min<size_t>(warm_bytes / 128, 1u << 24) : 0;
+               const int32_t* rows_dev, hipStream_t stream, const WarmList& warm) {
   int vec = 0, iters = 0;
   if (!ln_pick<T>(n, vec, iters)) return;
   // enough wavefronts to fill 256 CUs several times over; rows beyond that are looped
@@ -307,11 +309,11 @@ void ln_launch(void* out, const void* input, const void* bias, const void* gamma
   const T *i = (const T*)input, *b = (const T*)bias, *g = (const T*)gamma, *be = (const T*)beta;
   constexpr int MV = 16 / (int)sizeof(T);
   if (vec == MV)
-    ln_launch_iters<T, MV>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm, warm_lines);
+    ln_launch_iters<T, MV>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm);
   else if (vec == MV / 2)
-    ln_launch_iters<T, MV / 2>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm, warm_lines);
+    ln_launch_iters<T, MV / 2>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm);
   else
-    ln_launch_iters<T, MV / 4>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm, warm_lines);
+    ln_launch_iters<T, MV / 4>(iters, grid, stream, o, i, b, g, be, m, n, rows_dev, warm);
 }
 
 struct EmbedArgs {
@@ -391,13 +393,24 @@ bool bias_residual_layernorm_supported(DType t, int n) {
   return t == DType::F32 ? ln_pick<float>(n, vec, iters) : ln_pick<_Float16>(n, vec, iters);
 }
 
+void WarmList::add(const void* region, size_t bytes) {
+  // whole lines of a 128-byte aligned region; a list that is full or a region that is not aligned is left out
+  const size_t n = bytes / 128;
+  int slot = 0;
+  while (slot < kMax && lines[slot] != 0) ++slot;
+  if (region == nullptr || n == 0 || slot == kMax || ((uintptr_t)region & 127) != 0 || n + (size_t)total > (1u << 24)) return;
+  p[slot] = (const uint32_t*)region;
+  lines[slot] = (int)n;
+  total += (int)n;
+}
+
 void launch_bias_residual_layernorm(DType t, void* out, const void* input, const void* bias, const void* gamma,
                                     const void* beta, int m, int n, const int32_t* rows_dev, hipStream_t stream,
-                                    const void* warm_region, size_t warm_bytes) {
+                                    const WarmList& warm) {
   if (t == DType::F32)
-    ln_launch<float>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm_region, warm_bytes);
+    ln_launch<float>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm);
   else
-    ln_launch<_Float16>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm_region, warm_bytes);
+    ln_launch<_Float16>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm);
 }
 
 }  // namespace et

@@ -198,6 +198,7 @@ class LayerWeights:
             setattr(s, name, self.t[name].data_ptr())
         self.struct = s
         self.prepared: Optional[_lib.LayerPrepared] = None
+        self.warm_block: Optional[torch.Tensor] = None
         self._prepared_tensors: List[torch.Tensor] = []
 
     def prepare(self, every_kernel: bool = True) -> "LayerWeights":
@@ -217,10 +218,17 @@ class LayerWeights:
             names += [("attr_output_kernel", "attr_output_kernel_t"), ("output_kernel", "output_kernel_t")]
         self._prepared_tensors = []
         with torch.cuda.device(dev):
+            # the copies of Q, K, V and the attention output kernel lie one behind the other: one region for the layer in
+            # front of this one to request (et_layer_prepared.warm)
+            hq = self.t["attr_kernel_q"].shape[0]
+            together = [nm for nm, _ in names if nm.startswith("attr_") and tuple(self.t[nm].shape) == (hq, hq)]
+            block = torch.empty(len(together), hq, hq, dtype=torch.float16, device=dev)
+            self.warm_block = block if len(together) >= 3 else None
             for src_name, field in names:
                 src = self.t[src_name]
                 k, n = src.shape
-                dst = torch.empty(n, k, dtype=src.dtype, device=dev)
+                dst = block[together.index(src_name)] if src_name in together else \
+                    torch.empty(n, k, dtype=src.dtype, device=dev)
                 _lib.check(lib.et_transpose_weight(h, _lib.ET_FP16, _p(src), _p(dst), k, n, _stream()), h)
                 self._prepared_tensors.append(dst)
                 setattr(prep, field, dst.data_ptr())
@@ -354,6 +362,11 @@ class EffectiveTransformerEncoder:
         if prepare:
             for w in self.layers:
                 w.prepare()
+            # a layer's last kernel requests the next layer's attention weights, which would otherwise be read cold
+            for w, nxt in zip(self.layers[:-1], self.layers[1:]):
+                if w.prepared is not None and getattr(nxt, "warm_block", None) is not None:
+                    w.prepared.warm = nxt.warm_block.data_ptr()
+                    w.prepared.warm_bytes = nxt.warm_block.numel() * 2
         self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
 
     @classmethod

@@ -135,7 +135,11 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
  *        only.  Used where et_layer would run its large-M GEMM (it then skips its per-call transposition; Q, K and V
  *        go together); ignored for batches that run the small-M kernels, which read the [in,out] tensors.
  *   seq_start: the sequence table et_sequence_starts wrote for THIS batch (et_seq_workspace_bytes(batch_size) bytes);
- *        the same table serves every layer of the batch. */
+ *        the same table serves every layer of the batch.
+ *   warm, warm_bytes: a region that the layer's last kernel requests line by line on its way, so that whoever reads it
+ *        next finds it in the last-level cache: the k-contiguous copies of the NEXT layer's attention kernels, whose
+ *        GEMMs would otherwise wait for weights last read a whole batch ago.  Only used for batches large enough that
+ *        the region is small beside what that kernel moves anyway. */
 typedef struct et_layer_prepared {
   const void* attr_kernel_Q_t;       /* [H,H]  */
   const void* attr_kernel_K_t;       /* [H,H]  */
@@ -144,6 +148,8 @@ typedef struct et_layer_prepared {
   const void* inter_kernel_t;        /* [4H,H] */
   const void* output_kernel_t;       /* [H,4H] */
   const int32_t* seq_start;          /* [2B+1] */
+  const void* warm;                  /* see above; 128-byte aligned */
+  size_t warm_bytes;
 } et_layer_prepared;
 
 /* The sequence table of a batch, from the index arrays et_input produced: seq_start[b] = first packed row of sequence

@@ -78,7 +78,8 @@ class Encoder {
   Encoder(int device, et_dtype dtype, int head_num, int size_per_head, std::vector<et_layer_weights> layers,
           bool prepare = true)
       : handle_(device), dtype_(dtype), heads_(head_num), d_(size_per_head), layers_(std::move(layers)) {
-    prepared_.assign(layers_.size(), et_layer_prepared{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr});
+    prepared_.assign(layers_.size(),
+                     et_layer_prepared{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0});
     if (!prepare || dtype != ET_FP16) return;
     check_hip(hipSetDevice(device), "hipSetDevice");
     const size_t H = (size_t)head_num * size_per_head;
@@ -98,6 +99,12 @@ class Encoder {
       p.attr_output_kernel_t = transposed(w.attr_output_kernel, (int)H, (int)H);
       p.inter_kernel_t = transposed(w.inter_kernel, (int)H, (int)(4 * H));
       p.output_kernel_t = transposed(w.output_kernel, (int)(4 * H), (int)H);
+    }
+    // a layer's last kernel requests the next layer's Q/K/V and attention output copies (consecutive in wt_), which
+    // would otherwise be read cold
+    for (size_t l = 0; l + 1 < layers_.size(); ++l) {
+      prepared_[l].warm = prepared_[l + 1].attr_kernel_Q_t;
+      prepared_[l].warm_bytes = 4 * H * H * 2;
     }
     check_hip(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
   }
