@@ -506,8 +506,11 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   // attention weights (another -0.7 .. -1.6 % from 4000 to 40000 tokens, FFN-up included).
   const bool warm_fits = (double)rows * (7.0 * H + F) * (double)e <= kWarmLayerBytes;
   et::WarmList warm1, warm2;
-  if (t_up && rows >= F) warm1.add(wt_up, (size_t)H * F * e);
-  if (t_down && rows >= F && warm_fits) warm1.add(wt_down, (size_t)H * F * e);
+  // (whichever copy the GEMM reads, unless this call has just written it)
+  const void* b_up = t_up ? wt_up : w->inter_kernel;
+  const void* b_down = t_down ? wt_down : w->output_kernel;
+  if (rows >= F && !(t_up && !pp.inter_kernel_t)) warm1.add(b_up, (size_t)H * F * e);
+  if (rows >= F && warm_fits && !(t_down && !pp.output_kernel_t)) warm1.add(b_down, (size_t)H * F * e);
   if (rows >= F) warm2.add(pp.warm, pp.warm_bytes);
   et::launch_bias_residual_layernorm(dt, attn, from_tensor, w->attr_output_bias, w->attr_output_layernorm_gamma,
                                      w->attr_output_layernorm_beta, rows, H, T, st, warm1);

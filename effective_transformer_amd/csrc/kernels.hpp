@@ -123,7 +123,7 @@ bool gemm_blocked_handover(DType t, int m_bound, int wide, int narrow);
 // The large-M fp16 kernel is faster when B comes k-contiguous ([n][k]): both operands then reach the
 // MFMA with 128-bit LDS reads and no register transpose.  True when launch_gemm would use that kernel.
 bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
-// ... and where the encoder layer found the extra copy worth its time (measured inside the layer, not in isolation).
+// ... and where the encoder layer finds a per-call copy worth its time (everywhere it can be used).
 bool gemm_prefers_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups);
 // dst[j] ([n][k], row-major) = transpose of src[j] ([k][n], row-major), fp16, one launch for all jobs.
 struct TransposeJobs {
