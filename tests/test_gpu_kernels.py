@@ -369,8 +369,9 @@ def test_gemm(k, dtype, m, n, k_):
 # of 32 .. 128 rows by 64 .. 256 columns, with ragged last tiles in both directions and a single pair of k-steps.  The
 # last eighteen shapes reach, on a 256-CU part, every tile of that kernel in both of its ring depths: 32x64, 64x64,
 # 64x128, 96x64, 96x128, 96x192, 128x64, 128x128, 128x192 with a CU per workgroup and with two workgroups per CU, and
-# 128x256; three of the 192-column ones have a ragged last column tile.  The oracle product is taken on the CPU in
-# float64 for a sample of rows.
+# 128x256; three of the 192-column ones have a ragged last column tile.  The last shape is large enough (A and C
+# together above 128 MB) for the persistent kernel's non-temporal C stores; the persistent shapes before it take its
+# plain stores.  The oracle product is taken on the CPU in float64 for a sample of rows.
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072),
                                     (23301, 768, 768), (14000, 1032, 128),
                                     (13097, 768, 3072), (15866, 768, 768), (13097, 1024, 1024),
@@ -380,7 +381,7 @@ def test_gemm(k, dtype, m, n, k_):
                                     (5419, 768, 128), (1393, 768, 192), (3467, 776, 128), (2735, 768, 128),
                                     (6151, 768, 128), (5480, 768, 192), (9348, 776, 128), (1881, 776, 128),
                                     (4626, 776, 128), (4077, 768, 128), (8225, 776, 64), (3849, 1032, 192),
-                                    (9803, 776, 128), (8225, 768, 128)])
+                                    (9803, 776, 128), (8225, 768, 128), (40000, 1032, 640)])
 def test_gemm_bt(k, m, n, k_):
     print("gemm_bt", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_)
@@ -448,10 +449,12 @@ def test_gemm_bias_gelu_equals_the_two_passes(k, dtype, m, n, k_):
         k.gemm(dev(a), dev(b), gelu=True)
 
 
-# (the last four shapes: 192-column tiles, whose lanes store a group of four and a group of two columns)
+# (the four shapes before the last: 192-column tiles, whose lanes store a group of four and a group of two columns;
+# the last one: the persistent kernel's non-temporal stores behind the GELU)
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (5000, 3072, 768), (2000, 3072, 768),
                                     (1000, 776, 128), (400, 768, 768), (350, 200, 64),
-                                    (5480, 768, 128), (3849, 1032, 64), (9803, 776, 64), (1288, 3080, 64)])
+                                    (5480, 768, 128), (3849, 1032, 64), (9803, 776, 64), (1288, 3080, 64),
+                                    (36000, 1032, 768)])
 def test_gemm_bt_bias_gelu_equals_the_two_passes(k, m, n, k_):
     print("gemm_bt_bias_gelu", m, n, k_, flush=True)
     rng = np.random.RandomState(m + n + k_ + 1)
