@@ -834,6 +834,271 @@ void attention_long_launch(const void* q, const void* k, const void* v, int layo
 }
 
 // ------------------------------------------------------------------------------------------
+// fp16 fused attention for 128 < seq_len <= 512 with K and V of the whole sequence resident in LDS: one workgroup of
+// 8 wavefronts per (head, sequence) (or per share of its query tiles, see `qsplit`).  K and V are staged once (73 + 81
+// KB at 512 keys) instead of once per block of 64 queries, and after that one barrier the wavefronts run their
+// 16-query tiles independently: S^T = K Q^T over all key tiles, the softmax over the registers, O^T = V^T P^T.  The
+// arithmetic, its order and the rounding points are those of attention_long_kernel (the results are the same bits).
+// ------------------------------------------------------------------------------------------
+constexpr int kResThreads = 512;
+constexpr int kResWaves = kResThreads / kWave;
+
+template <int NKT>
+struct ResSmem {
+  static constexpr int kSp = NKT * 16;
+  static constexpr int kQS = AttnCfg<_Float16>::kQkStride;
+  static constexpr int kVR = AttnCfg<_Float16>::kVStride;
+  static constexpr size_t kKBytes = (size_t)kSp * kQS * 2;
+  static constexpr size_t kVBytes = (size_t)kSp * kVR * 2;
+  static constexpr size_t kBytes = kKBytes + kVBytes + (size_t)kSp * sizeof(int);
+};
+
+template <int NKT>
+__global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(NKT <= 16 ? 4 : 2, NKT <= 16 ? 4 : 2)))
+void attention_resident_kernel(
+    const _Float16* __restrict__ q_src, const _Float16* __restrict__ k_src, const _Float16* __restrict__ v_src, int layout,
+    int packed_ld, const _Float16* __restrict__ attr_mask, _Float16* __restrict__ dst,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads,
+    int qsplit, float scaler) {
+  using T = _Float16;
+  using Sm = ResSmem<NKT>;
+  using C = Chunk16<T>;
+  using V16 = typename C::vec;
+  constexpr int kQS = Sm::kQS, kVR = Sm::kVR, kSp = Sm::kSp;
+  constexpr int kCpr = kD / C::kElems;                       // 16-byte pieces per head row
+  typedef T mask4 __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* Ks = reinterpret_cast<T*>(smem_raw);
+  T* Vs = reinterpret_cast<T*>(smem_raw + Sm::kKBytes);
+  int* tok_of_pos = reinterpret_cast<int*>(smem_raw + Sm::kKBytes + Sm::kVBytes);
+
+  const int b = min(max(seq_start[batch + 1 + blockIdx.y], 0), batch - 1);
+  const int head = blockIdx.x / qsplit, part = blockIdx.x - head * qsplit;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  const int len = t1 - t0;
+  if (len <= 0) return;
+  const int H = heads * kD;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int l16 = lane & 15, g = lane >> 4;
+
+  const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
+  const int n_tiles = last_pos / 16 + 1;                     // 16-row tiles that hold at least one token
+  if (part >= n_tiles) return;                               // no query tile for this share (workgroup-uniform)
+  for (int i = threadIdx.x; i < kSp; i += kResThreads) tok_of_pos[i] = -1;
+  __syncthreads();
+  for (int tt = threadIdx.x; tt < len; tt += kResThreads) {
+    const int pos = word_idx[t0 + tt];
+    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = t0 + tt;
+  }
+  __syncthreads();
+
+  auto src_off = [&](int t, int pos) -> size_t {
+    return layout == 1 ? (size_t)t * packed_ld + head * kD : (((size_t)b * heads + head) * seq_len + pos) * kD;
+  };
+  // K and V rows of every group of four key tiles that holds a token (the loops below run over such groups), zeros
+  // where no token sits; four pieces of each per thread in flight
+  {
+    const int rows = min(kSp, ((n_tiles + 3) / 4) * 64);
+    const int pieces = rows * kCpr;
+    constexpr int kFly = 4;
+    for (int i0 = threadIdx.x; i0 < pieces; i0 += kFly * kResThreads) {
+      V16 rk[kFly], rv[kFly];
+#pragma unroll
+      for (int u = 0; u < kFly; ++u) {
+        const int i = i0 + u * kResThreads;
+        const int row = i / kCpr, c = i - row * kCpr;
+#pragma unroll
+        for (int j = 0; j < C::kElems; ++j) {
+          rk[u][j] = (T)0;
+          rv[u][j] = (T)0;
+        }
+        const int tk = i < pieces ? tok_of_pos[row] : -1;
+        if (tk >= 0) {
+          const size_t off = src_off(tk, row) + c * C::kElems;
+          rk[u] = *reinterpret_cast<const V16*>(k_src + off);
+          rv[u] = *reinterpret_cast<const V16*>(v_src + off);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kFly; ++u) {
+        const int i = i0 + u * kResThreads;
+        if (i < pieces) {
+          const int row = i / kCpr, c = i - row * kCpr;
+          *reinterpret_cast<V16*>(Ks + row * kQS + c * C::kElems) = rk[u];
+          *reinterpret_cast<V16*>(Vs + row * kVR + c * C::kElems) = rv[u];
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  const bool vec_mask = (seq_len & 3) == 0;
+  for (int qt = part + qsplit * wave; qt < n_tiles; qt += qsplit * kResWaves) {
+    const int q = qt * 16 + l16;
+    const int tq = tok_of_pos[q];
+    const T* mrow = attr_mask + ((size_t)b * seq_len + min(q, seq_len - 1)) * seq_len;
+    // Q operand of this lane (zeros for a query position without a token: its result is never stored)
+    half8 bqh[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bqh[ks][j] = (_Float16)0;
+      if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + src_off(tq, q) + ks * 32 + g * 8);
+    }
+
+    // ---- the additive bias of the mask row first: no branch between its loads, eight in flight ------------------
+    float s[NKT][4];
+    const int n_groups = (n_tiles + 3) / 4;
+    // (opaque to the compiler, or it would keep the clamped offsets of all key tiles in registers across query tiles)
+    int g4 = g * 4;
+    asm volatile("" : "+v"(g4));
+    if (vec_mask) {
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        const int key0 = kt * 16 + g4;
+        const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + min(key0, seq_len - 4));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] = key0 < seq_len ? (1.0f - (float)m4[r]) * -10000.0f : -INFINITY;
+        if (kt % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        const int key0 = kt * 16 + g4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const T m = mrow[min(key0 + r, seq_len - 1)];
+          s[kt][r] = key0 + r < seq_len ? (1.0f - (float)m) * -10000.0f : -INFINITY;
+        }
+        if (kt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- S^T = K Q^T, four key tiles at a time (rows without a token are zero: score 0) ---------------------
+#pragma unroll
+    for (int kg = 0; kg < NKT / 4; ++kg) {
+      if (kg < n_groups) {
+#pragma unroll
+        for (int kc = 0; kc < 4; ++kc) {
+          const int kt = kg * 4 + kc;
+          float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks) {
+            const half8 a = *reinterpret_cast<const half8*>(Ks + (kt * 16 + l16) * kQS + ks * 32 + g * 8);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bqh[ks], acc, 0, 0, 0);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float sc = h2f(f2h(acc[r]));                         // the score is stored in half
+            s[kt][r] = sc * scaler + s[kt][r];                         // -inf stays -inf for keys that do not exist
+          }
+        }
+      }
+    }
+
+    // ---- masked softmax over the registers ------------------------------------------------------------
+    {
+      float mx = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][r]);
+      mx = xor_lanes_16_32_max(mx) * kLog2e;
+      float sum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          s[kt][r] = __builtin_amdgcn_exp2f(s[kt][r] * kLog2e - mx);
+          sum += s[kt][r];
+        }
+      sum = xor_lanes_16_32_sum(sum) + 1e-6f;
+      const float inv = 1.0f / sum;
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
+    }
+
+    // ---- O^T = V^T P^T over pairs of key tiles ----------------------------------------------------------
+    float4v o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kp = 0; kp < NKT / 2; ++kp) {
+      const int kt = 2 * kp;
+      if (kp / 2 < n_groups) {
+        half8 p;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[r] = f2h(s[kt][r]);
+          p[4 + r] = f2h(s[kt + 1][r]);
+        }
+        typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u2 raw[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          const int key = kp * 32 + (kk >> 2) * 16 + g * 4 + (kk & 3);
+          raw[kk] = *reinterpret_cast<const u2*>(Vs + key * kVR + l16 * 4);
+        }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          u4 lo, hi;
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            lo[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x05040100u);
+            hi[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x07060302u);
+          }
+          o[2 * jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, lo), p, o[2 * jj], 0, 0, 0);
+          o[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, hi), p, o[2 * jj + 1], 0, 0, 0);
+        }
+      }
+    }
+
+    if (tq >= 0) {
+      half8 v0, v1;
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v0[4 * r + j] = f2h(o[j][r]);
+          v1[4 * r + j] = f2h(o[j][2 + r]);
+        }
+      T* orow = dst + (size_t)tq * H + head * kD + g * 16;
+      *reinterpret_cast<half8*>(orow) = v0;
+      *reinterpret_cast<half8*>(orow + 8) = v1;
+    }
+  }
+}
+
+inline int attention_cu_count() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    return 256;
+  return n;
+}
+
+template <int NKT>
+void attention_resident_launch(const void* q, const void* k, const void* v, int layout, int packed_ld,
+                               const void* attr_mask, void* dst, const int32_t* seq_start, const int32_t* word_idx,
+                               int batch, int seq_len, int heads, float scaler, hipStream_t stream) {
+  using Sm = ResSmem<NKT>;
+  auto kern = attention_resident_kernel<NKT>;
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Sm::kBytes);
+  // few (head, sequence) pairs: the query tiles of a pair are dealt to 2 or 4 workgroups, each staging K and V itself
+  const long pairs = (long)heads * batch;
+  const int cus = attention_cu_count();
+  const int qsplit = pairs >= cus ? 1 : (2 * pairs >= cus ? 2 : 4);
+  dim3 grid(heads * qsplit, batch);
+  kern<<<grid, kResThreads, Sm::kBytes, stream>>>((const _Float16*)q, (const _Float16*)k, (const _Float16*)v, layout,
+                                                 packed_ld, (const _Float16*)attr_mask, (_Float16*)dst, seq_start,
+                                                 word_idx, batch, seq_len, heads, qsplit, scaler);
+}
+
+// ------------------------------------------------------------------------------------------
 // fused attention for every shape the MFMA kernels above are not built for: size_per_head other than 64 (any
 // multiple of 16 bytes up to 256 elements) and 512 < seq_len <= 1024.  One wavefront per (query, head): the lanes
 // split the keys for the scores (full dot products in float, rounded to the element type as the reference stores
@@ -965,6 +1230,15 @@ void attention_dispatch(const void* q, const void* k, const void* v, int layout,
   if (d != kD || seq_len > 512)
     attention_generic_launch<T>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads, d,
                                 scaler, stream);
+  else if (sizeof(T) == 2 && seq_len > 384)
+    attention_resident_launch<32>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                                  scaler, stream);
+  else if (sizeof(T) == 2 && seq_len > 256)
+    attention_resident_launch<24>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                                  scaler, stream);
+  else if (sizeof(T) == 2 && seq_len > 128)
+    attention_resident_launch<16>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                                  scaler, stream);
   else if (seq_len > 256)
     attention_long_launch<T, 32>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
                                  scaler, stream);

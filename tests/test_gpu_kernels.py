@@ -243,7 +243,8 @@ def test_softmax(k, dtype, S):
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 @pytest.mark.parametrize("S,holes,weird", [(5, False, False), (32, False, False), (64, False, False),
                                            (64, True, True), (100, True, False), (128, False, True), (21, True, True),
-                                           # beyond 128 positions: the chunked kernel (K and V in 128-key chunks)
+                                           # beyond 128 positions: fp32 the chunked kernel (K and V in 128-key chunks),
+                                           # fp16 the kernel that keeps K and V of a sequence in LDS
                                            (129, False, False), (200, True, True), (256, False, False),
                                            (300, True, False), (384, False, True), (512, False, False), (509, True, True)])
 def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
@@ -276,6 +277,31 @@ def test_fused_attention_both_layouts(k, dtype, S, holes, weird):
     else:
         # fp32 accumulation vs the oracle's exact sums, three roundings to half on the way
         np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
+
+
+# fp16, 128 < seq_len <= 512: K and V of a sequence stay in LDS for all of its query tiles, which are dealt to one, two
+# or four workgroups per (head, sequence) depending on how many such pairs the batch has (on a 256-CU part: 288, 144
+# and 12 pairs here).
+@pytest.mark.parametrize("B,heads,S,holes,weird", [(24, 12, 200, True, False), (12, 12, 300, False, True),
+                                                   (3, 4, 500, True, True), (22, 12, 130, False, False)])
+def test_fused_attention_with_resident_keys(k, B, heads, S, holes, weird):
+    print("attention resident", B, heads, S, holes, weird, flush=True)
+    p = _attn_problem(B + S, B, S, heads, "fp16", holes=holes, weird_mask=weird)
+    bi, wi, vwn = _idx_dev(p)
+    T, d = p["T"], p["d"]
+    H = heads * d
+    qp, kp, vp = o.add_qkv_bias_padding(p["q"], p["bq"], p["k"], p["bk"], p["v"], p["bv"], T, B, S, heads, d, p["bi"],
+                                        p["wi"], "fp16")
+    want = o.attention(qp, kp, vp, p["attr"], T, p["bi"], p["wi"], "fp16")
+    got0 = k.attention(dev(qp), dev(kp), dev(vp), 0, 0, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    packed = np.zeros((B * S, 3 * H), np.float16)
+    packed[:T, :H] = o.hadd(p["q"], p["bq"]); packed[:T, H:2 * H] = o.hadd(p["k"], p["bk"])
+    packed[:T, 2 * H:] = o.hadd(p["v"], p["bv"])
+    pk = dev(packed)
+    got1 = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(p["attr"]), vwn, B, S, heads, d, bi, wi).cpu().numpy()
+    assert np.array_equal(got0, got1)
+    assert np.all(got0[T:] == 0)
+    np.testing.assert_allclose(got0[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
