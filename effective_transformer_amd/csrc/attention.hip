@@ -954,13 +954,24 @@ void attention_resident_kernel(
     // (opaque to the compiler, or it would keep the clamped offsets of all key tiles in registers across query tiles)
     int g4 = g * 4;
     asm volatile("" : "+v"(g4));
-    if (vec_mask) {
+    // (1 - m) * -10000 as one fma: 1 - m is exact in float for a half m, so both forms round the same real number once
+    if (seq_len == kSp) {
+      // every key of every tile exists
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt) {
+        const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + kt * 16 + g4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] = __builtin_fmaf((float)m4[r], 10000.0f, -10000.0f);
+        if (kt % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+      }
+    } else if (vec_mask) {
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt) {
         const int key0 = kt * 16 + g4;
         const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + min(key0, seq_len - 4));
 #pragma unroll
-        for (int r = 0; r < 4; ++r) s[kt][r] = key0 < seq_len ? (1.0f - (float)m4[r]) * -10000.0f : -INFINITY;
+        for (int r = 0; r < 4; ++r)
+          s[kt][r] = key0 < seq_len ? __builtin_fmaf((float)m4[r], 10000.0f, -10000.0f) : -INFINITY;
         if (kt % 8 == 7) __builtin_amdgcn_sched_barrier(0);
       }
     } else {
@@ -970,7 +981,7 @@ void attention_resident_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const T m = mrow[min(key0 + r, seq_len - 1)];
-          s[kt][r] = key0 + r < seq_len ? (1.0f - (float)m) * -10000.0f : -INFINITY;
+          s[kt][r] = key0 + r < seq_len ? __builtin_fmaf((float)m, 10000.0f, -10000.0f) : -INFINITY;
         }
         if (kt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
       }
