@@ -363,10 +363,12 @@ class EffectiveTransformerEncoder:
             for w in self.layers:
                 w.prepare()
             # a layer's last kernel requests the next layer's attention weights, which would otherwise be read cold
+            self._warm_refs = []         # the regions named below stay allocated as long as this encoder lives
             for w, nxt in zip(self.layers[:-1], self.layers[1:]):
                 if w.prepared is not None and getattr(nxt, "warm_block", None) is not None:
                     w.prepared.warm = nxt.warm_block.data_ptr()
                     w.prepared.warm_bytes = nxt.warm_block.numel() * 2
+                    self._warm_refs.append(nxt.warm_block)
         self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
 
     @classmethod
