@@ -58,7 +58,7 @@ namespace {
 // stores beyond.  12-layer BERT-base, fp16: plain stores -6 % at 4000 tokens, -2.4 % at 15900, +-0.5 % at 20000,
 // +2 % at 30000 and 40000; 24-layer BERT-large at 13100 tokens: -0.4 %.
 constexpr double kCachedLayerBytes = 320.0 * 1048576.0;
-constexpr double kCachedCallBytes = 128.0 * 1048576.0;
+constexpr double kCachedCallBytes = 96.0 * 1048576.0;
 constexpr double kWarmLayerBytes = 256.0 * 1048576.0;
 constexpr int kStaticScratchWords = 1024;
 constexpr int kStaticMaxPositions = 1024 * 1024;

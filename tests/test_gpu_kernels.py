@@ -396,7 +396,7 @@ def test_gemm(k, dtype, m, n, k_):
 # last eighteen shapes reach, on a 256-CU part, every tile of that kernel in both of its ring depths: 32x64, 64x64,
 # 64x128, 96x64, 96x128, 96x192, 128x64, 128x128, 128x192 with a CU per workgroup and with two workgroups per CU, and
 # 128x256; three of the 192-column ones have a ragged last column tile.  The last shape is large enough (A and C
-# together above 128 MB) for the persistent kernel's non-temporal C stores; the persistent shapes before it take its
+# together above 96 MB) for the persistent kernel's non-temporal C stores; the persistent shapes before it take its
 # plain stores.  The oracle product is taken on the CPU in float64 for a sample of rows.
 @pytest.mark.parametrize("m,n,k_", [(11000, 768, 768), (8200, 1032, 128), (4100, 2304, 768), (10900, 776, 3072),
                                     (23301, 768, 768), (14000, 1032, 128),
