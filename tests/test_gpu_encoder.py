@@ -330,7 +330,8 @@ def test_long_sequences_layer_against_oracle(dtype):
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 @pytest.mark.parametrize("B,S,heads,d", [(4, 48, 4, 32), (3, 40, 2, 128), (2, 600, 2, 64), (1, 1024, 1, 64), (2, 520, 4, 32),
-                                         (5, 40, 3, 32)])      # hidden size 96: no multiple of 64, the weights stay [k][n]
+                                         (5, 40, 3, 32),       # hidden size 96: no multiple of 64, the weights stay [k][n]
+                                         (3, 384, 2, 64), (2, 512, 12, 64), (4, 250, 3, 64)])  # keys resident in LDS (fp16)
 def test_other_head_sizes_and_sequences_beyond_512(dtype, B, S, heads, d):
     """The reference op takes any size_per_head (tf_op/bert_transformer_op.cc:53-57) and sequences up to the 1024 keys
     its softmax launcher covers (cuda/attention.cu:345-356): one layer against the oracle."""
