@@ -1110,6 +1110,372 @@ void attention_resident_launch(const void* q, const void* k, const void* v, int 
 }
 
 // ------------------------------------------------------------------------------------------
+// fused attention for 512 < seq_len <= 1024: the chunked kernel above with the keys of a query tile split over two
+// wavefronts.  One workgroup of 8 wavefronts per (64 queries, head, sequence): wavefront w serves query tile w & 3 and
+// the key half w >> 2 (512 keys: 4 scores per lane and key tile, 128 VGPRs).  K and V pass through LDS in chunks of
+// 128 keys per half, both halves in the same step.  The two halves of a query tile exchange their maxima and their
+// sums through LDS (sum = first half + second half, the same on both sides), and the second half hands its part of
+// O over for the first to add and store.  Arithmetic and rounding points per element are those of the other kernels;
+// at 1024 keys the maximum is not clamped at 0 (see attention_generic_kernel).
+// ------------------------------------------------------------------------------------------
+constexpr int kSplitThreads = 512;
+constexpr int kSplitHalfTiles = 32;               // key tiles per wavefront
+constexpr int kSplitKeys = 2 * kSplitHalfTiles * 16;
+
+template <typename T>
+__global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
+    const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
+    const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, float scaler) {
+  using Sm = LongSmem<T>;
+  using C = Chunk16<T>;
+  using V16 = typename C::vec;
+  constexpr int kQS = Sm::kQS, kVR = Sm::kVR, kVS = Sm::kVS;
+  constexpr int kCpr = kD / C::kElems;
+  constexpr int NKT = kSplitHalfTiles;
+  constexpr int kChunks = NKT / kLongChunkTiles;             // 4 steps of 128 keys per half
+  constexpr int CPT = kLongChunk * kCpr / kAttnThreads;      // 16-byte pieces of a chunk per thread of a half
+  typedef T mask4 __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  int* tok_of_pos = reinterpret_cast<int*>(smem_raw + 2 * Sm::kTileBytes);
+  float* red = reinterpret_cast<float*>(smem_raw + 2 * Sm::kTileBytes + kSplitKeys * sizeof(int));   // [2][4 tiles][2 halves][16]
+
+  const int b = min(max(seq_start[batch + 1 + blockIdx.z], 0), batch - 1), head = blockIdx.y, qblock = blockIdx.x;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  const int len = t1 - t0;
+  if (len <= 0) return;
+  const int H = heads * kD;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int tile_w = wave & 3, half = wave >> 2;
+  const int l16 = lane & 15, g = lane >> 4;
+  // this half's staging threads (256 per half) and its chunk buffer
+  const int tid_h = threadIdx.x & (kAttnThreads - 1);
+  T* Ks = reinterpret_cast<T*>(smem_raw + half * Sm::kTileBytes);
+  T* Vs = Ks;
+  const int kt_base = half * NKT;                            // first key tile of this half
+
+  const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
+  const int n_tiles = last_pos / 16 + 1;                     // 16-row tiles that hold at least one token
+  if (qblock * 4 >= n_tiles) return;                         // no token among this workgroup's queries
+  for (int i = threadIdx.x; i < kSplitKeys; i += kSplitThreads) tok_of_pos[i] = -1;
+  __syncthreads();
+  for (int tt = threadIdx.x; tt < len; tt += kSplitThreads) {
+    const int pos = word_idx[t0 + tt];
+    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = t0 + tt;
+  }
+  __syncthreads();
+
+  auto src_off = [&](int t, int pos) -> size_t {
+    return layout == 1 ? (size_t)t * packed_ld + head * kD : (((size_t)b * heads + head) * seq_len + pos) * kD;
+  };
+  // rows [c0, c0 + 128) of `src`, zeros where no token sits: global memory -> registers, registers -> this half's
+  // buffer (row-major, stride `stride` elements).  The fp16 kernel fetches a chunk while the one before it is used.
+  auto fetch_rows = [&](const T* __restrict__ src, int c0, V16 (&r)[CPT]) {
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+      const int i = tid_h + k * kAttnThreads;
+      const int row = i / kCpr, c = i - row * kCpr;
+      const int pos = c0 + row;
+      const int tk = pos < kSplitKeys ? tok_of_pos[pos] : -1;
+#pragma unroll
+      for (int j = 0; j < C::kElems; ++j) r[k][j] = (T)0;
+      if (tk >= 0) r[k] = *reinterpret_cast<const V16*>(src + src_off(tk, pos) + c * C::kElems);
+    }
+  };
+  auto put_rows = [&](T* lds, int stride, const V16 (&r)[CPT]) {
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+      const int i = tid_h + k * kAttnThreads;
+      const int row = i / kCpr, c = i - row * kCpr;
+      *reinterpret_cast<V16*>(lds + row * stride + c * C::kElems) = r[k];
+    }
+  };
+  auto stage_rows = [&](const T* __restrict__ src, T* lds, int stride, int c0) {
+    V16 r[CPT];
+    fetch_rows(src, c0, r);
+    put_rows(lds, stride, r);
+  };
+  constexpr bool kAhead = sizeof(T) == 2;                    // fp32: twice the registers per chunk, no room
+  auto half_has_tokens = [&](int ch) { return kt_base + ch * kLongChunkTiles < n_tiles; };
+  V16 pre[kAhead ? CPT : 1];
+
+  const int qt = qblock * 4 + tile_w;                        // this wavefront's 16-query tile
+  const bool active = qt < n_tiles;                          // wave-uniform
+  const int q = qt * 16 + l16;
+  const int tq = (active && q < kSplitKeys) ? tok_of_pos[q] : -1;
+  const T* mrow = attr_mask + ((size_t)b * seq_len + min(q, seq_len - 1)) * seq_len;
+  const bool vec_mask = (seq_len & 3) == 0;
+
+  // Q operand of this lane (zeros for a query position without a token: its result is never stored)
+  half8 bqh[2];
+  float bqf[16];
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bqh[ks][j] = (_Float16)0;
+      if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + src_off(tq, q) + ks * 32 + g * 8);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float4v v4 = {0.f, 0.f, 0.f, 0.f};
+      if (tq >= 0) v4 = *reinterpret_cast<const float4v*>(q_src + src_off(tq, q) + g * 16 + i * 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bqf[i * 4 + j] = v4[j];
+    }
+  }
+
+  if constexpr (kAhead) {
+    if (half_has_tokens(0)) fetch_rows(k_src, kt_base * 16, pre);
+  }
+
+  // ---- the additive bias of this half of the mask row (no branch between the loads) -------------------------
+  float s[NKT][4];
+  {
+    int g4 = g * 4;
+    asm volatile("" : "+v"(g4));       // opaque: the clamped offsets are recomputed, not kept in registers
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) {
+      const int key0 = (kt_base + kt) * 16 + g4;
+      if (vec_mask) {
+        const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + min(key0, seq_len - 4));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kt][r] = key0 < seq_len ? (1.0f - (float)m4[r]) * -10000.0f : -INFINITY;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const T m = mrow[min(key0 + r, seq_len - 1)];
+          s[kt][r] = key0 + r < seq_len ? (1.0f - (float)m) * -10000.0f : -INFINITY;
+        }
+      }
+      if (kt % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- S^T = K Q^T chunk by chunk -------------------------------------------------------------------------
+#pragma unroll
+  for (int ch = 0; ch < kChunks; ++ch) {
+    if (ch * kLongChunkTiles >= n_tiles) break;                          // workgroup-uniform: no token in either half
+    const bool chunk_has_tokens = kt_base + ch * kLongChunkTiles < n_tiles;   // uniform over this half's 4 wavefronts
+    __syncthreads();                                                     // previous chunks fully consumed
+    if (chunk_has_tokens) {
+      if constexpr (kAhead) {
+        put_rows(Ks, kQS, pre);
+      } else {
+        stage_rows(k_src, Ks, kQS, (kt_base + ch * kLongChunkTiles) * 16);
+      }
+    }
+    __syncthreads();
+    if constexpr (kAhead) {
+      if (ch + 1 < kChunks && half_has_tokens(ch + 1))
+        fetch_rows(k_src, (kt_base + (ch + 1) * kLongChunkTiles) * 16, pre);
+      else if (half_has_tokens(0) && (ch + 1 == kChunks || (ch + 1) * kLongChunkTiles >= n_tiles))
+        fetch_rows(v_src, kt_base * 16, pre);                            // last K chunk of the workgroup: V comes next
+    }
+    if (active && chunk_has_tokens) {
+#pragma unroll
+      for (int kc = 0; kc < kLongChunkTiles; ++kc) {
+        const int ktl = ch * kLongChunkTiles + kc;
+        if (kt_base + ktl < n_tiles) {
+          float4v acc = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+              const half8 a = *reinterpret_cast<const half8*>(Ks + (kc * 16 + l16) * kQS + ks * 32 + g * 8);
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bqh[ks], acc, 0, 0, 0);
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kc * 16 + l16) * kQS + g * 16 + i * 4);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bqf[i * 4 + j], acc, 0, 0, 0);
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float sc = sizeof(T) == 2 ? h2f(f2h(acc[r])) : acc[r];   // the score is stored in the element type
+            s[ktl][r] = sc * scaler + s[ktl][r];
+          }
+        }
+      }
+    }
+  }
+
+  // ---- masked softmax: each half over its registers, maxima and sums exchanged through LDS --------------------
+  float* red_max = red;
+  float* red_sum = red + 4 * 2 * 16;
+  {
+    float mx = seq_len < kSplitKeys ? 0.f : -INFINITY;       // the clamp at 0 holds below 1024 keys
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][r]);
+    mx = xor_lanes_16_32_max(mx);
+    if (g == 0) red_max[(tile_w * 2 + half) * 16 + l16] = mx;
+  }
+  __syncthreads();
+  float inv;
+  {
+    const float mx = fmaxf(red_max[(tile_w * 2) * 16 + l16], red_max[(tile_w * 2 + 1) * 16 + l16]) * kLog2e;
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[kt][r] = __builtin_amdgcn_exp2f(s[kt][r] * kLog2e - mx);
+        sum += s[kt][r];
+      }
+    sum = xor_lanes_16_32_sum(sum);
+    if (g == 0) red_sum[(tile_w * 2 + half) * 16 + l16] = sum;
+  }
+  __syncthreads();
+  {
+    const float sum = red_sum[(tile_w * 2) * 16 + l16] + red_sum[(tile_w * 2 + 1) * 16 + l16] + 1e-6f;
+    inv = 1.0f / sum;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
+  }
+
+  // ---- O^T = V^T P^T chunk by chunk, each half over its keys ---------------------------------------------------
+  float4v o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ch = 0; ch < kChunks; ++ch) {
+    if (ch * kLongChunkTiles >= n_tiles) break;                         // workgroup-uniform
+    const bool chunk_has_tokens = kt_base + ch * kLongChunkTiles < n_tiles;
+    __syncthreads();
+    if (chunk_has_tokens) {
+      if constexpr (kAhead) {
+        put_rows(Vs, kVR, pre);
+      } else {
+        // fp32 keeps V^T: feature rows, key columns
+#pragma unroll
+        for (int k = 0; k < CPT; ++k) {
+          const int i = tid_h + k * kAttnThreads;
+          const int row = i / kCpr, c = i - row * kCpr;
+          const int pos = (kt_base + ch * kLongChunkTiles) * 16 + row;
+          const int tk = pos < kSplitKeys ? tok_of_pos[pos] : -1;
+          V16 r = {0.f, 0.f, 0.f, 0.f};
+          if (tk >= 0) r = *reinterpret_cast<const V16*>(v_src + src_off(tk, pos) + c * C::kElems);
+#pragma unroll
+          for (int j = 0; j < C::kElems; ++j) Vs[(c * C::kElems + j) * kVS + row] = r[j];
+        }
+      }
+    }
+    __syncthreads();
+    if constexpr (kAhead) {
+      if (ch + 1 < kChunks && half_has_tokens(ch + 1)) fetch_rows(v_src, (kt_base + (ch + 1) * kLongChunkTiles) * 16, pre);
+    }
+    if (!active || !chunk_has_tokens) continue;
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int kp = 0; kp < kLongChunkTiles / 2; ++kp) {
+        const int ktl = ch * kLongChunkTiles + 2 * kp;
+        if (kt_base + ktl < n_tiles) {
+          half8 p;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            p[r] = f2h(s[ktl][r]);
+            p[4 + r] = f2h(s[ktl + 1][r]);
+          }
+          typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+          typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+          u2 raw[8];
+#pragma unroll
+          for (int kk = 0; kk < 8; ++kk) {
+            const int key = kp * 32 + (kk >> 2) * 16 + g * 4 + (kk & 3);
+            raw[kk] = *reinterpret_cast<const u2*>(Vs + key * kVR + l16 * 4);
+          }
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            u4 lo, hi;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+              lo[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x05040100u);
+              hi[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x07060302u);
+            }
+            o[2 * jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, lo), p, o[2 * jj], 0, 0, 0);
+            o[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, hi), p, o[2 * jj + 1], 0, 0, 0);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int kc = 0; kc < kLongChunkTiles; ++kc) {
+        const int ktl = ch * kLongChunkTiles + kc;
+        if (kt_base + ktl < n_tiles) {
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) {
+            const float4v a4 = *reinterpret_cast<const float4v*>(Vs + (dt * 16 + l16) * kVS + kc * 16 + g * 4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[ktl][r], o[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- the second half hands its part of O over (through the chunk buffers, free now), the first adds and stores --
+  __syncthreads();
+  float4v* xo = reinterpret_cast<float4v*>(smem_raw);        // [4 tiles][64 lanes][4]
+  if (half == 1) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) xo[(tile_w * kWave + lane) * 4 + dt] = o[dt];
+  }
+  __syncthreads();
+  if (half == 0 && tq >= 0) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      const float4v other = xo[(tile_w * kWave + lane) * 4 + dt];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] += other[r];
+    }
+    if constexpr (sizeof(T) == 2) {
+      half8 v0, v1;
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v0[4 * r + j] = f2h(o[j][r]);
+          v1[4 * r + j] = f2h(o[j][2 + r]);
+        }
+      T* orow = dst + (size_t)tq * H + head * kD + g * 16;
+      *reinterpret_cast<half8*>(orow) = v0;
+      *reinterpret_cast<half8*>(orow + 8) = v1;
+    } else {
+      T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        float4v v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = o[dt][r];
+        *reinterpret_cast<float4v*>(orow + dt * 16) = v;
+      }
+    }
+  }
+}
+
+template <typename T>
+void attention_split_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
+                            void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
+                            float scaler, hipStream_t stream) {
+  const size_t smem = 2 * LongSmem<T>::kTileBytes + (size_t)kSplitKeys * sizeof(int) + 2 * 4 * 2 * 16 * sizeof(float);
+  auto kern = attention_split_kernel<T>;
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem);
+  dim3 grid(kSplitKeys / 64, heads, batch);
+  kern<<<grid, kSplitThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
+                                              (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch, seq_len, heads,
+                                              scaler);
+}
+
+// ------------------------------------------------------------------------------------------
 // fused attention for every shape the MFMA kernels above are not built for: size_per_head other than 64 (any
 // multiple of 16 bytes up to 256 elements) and 512 < seq_len <= 1024.  One wavefront per (query, head): the lanes
 // split the keys for the scores (full dot products in float, rounded to the element type as the reference stores
@@ -1238,9 +1604,12 @@ template <typename T>
 void attention_dispatch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                         void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                         int d, float scaler, hipStream_t stream) {
-  if (d != kD || seq_len > 512)
+  if (d != kD)
     attention_generic_launch<T>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads, d,
                                 scaler, stream);
+  else if (seq_len > 512)
+    attention_split_launch<T>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
+                              scaler, stream);
   else if (sizeof(T) == 2 && seq_len > 384)
     attention_resident_launch<32>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads,
                                   scaler, stream);
