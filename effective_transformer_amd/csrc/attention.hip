@@ -1462,14 +1462,292 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// fp16, 512 < seq_len <= 1024: the split kernel above with K of the whole sequence in LDS at once, then V in its place.
+// The score registers allow one workgroup per CU either way, so the workgroup takes 128 KB of LDS: every K row (128
+// bytes) arrives by DMA, all requests in flight together with the mask row and Q, instead of chunk after chunk through
+// registers with a fetch latency each; V follows into the same rows while the softmax runs.  A row without a token is
+// requested beyond its buffer descriptor's range and arrives as zeros.
+// Which key a row of an MFMA tile stands for is free as long as K, the mask and V agree: row m of the first tile of a
+// pair (32 keys from `base`) is key base + (m >> 2) * 8 + (m & 3), of the second tile 4 keys further.  A lane's scores
+// of a pair are then 8 consecutive keys: one 16-byte load of its mask row, and the P operand of the P.V MFMA is in
+// natural key order.  Key row `key` lies in slot key ^ ((key >> 3) & 1) (the two rows of a half-wave of the 8-byte V
+// reads, 8 keys apart, land on different halves of the banks), and the 16-byte chunks of a slot are XOR-swizzled with
+// slot bits 1, 3 and 4 (the 16 rows x one chunk of a K operand read cover all 64 banks).  Arithmetic and rounding
+// points per element are those of the split kernel.
+// ------------------------------------------------------------------------------------------
+constexpr int kWideKvBytes = kSplitKeys * 128;
+constexpr int kWideSmem = kWideKvBytes + kSplitKeys * (int)sizeof(int) + 2 * 4 * 2 * 16 * (int)sizeof(float);
+#define ET_ATTN_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+__device__ __forceinline__ int wide_slot(int key) { return key ^ ((key >> 3) & 1); }
+__device__ __forceinline__ int wide_swizzle(int slot) { return ((slot >> 1) & 1) | ((slot >> 2) & 6); }
+// s_waitcnt immediates of gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+__device__ __forceinline__ void wide_wait_dma() { __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8) | (0 << 14)); }
+__device__ __forceinline__ void wide_wait_lds() { __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14)); }
+// barrier without the fence of __syncthreads(), which would wait for every DMA in flight
+__device__ __forceinline__ void wide_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+__global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
+    const _Float16* __restrict__ q_src, const _Float16* __restrict__ k_src, const _Float16* __restrict__ v_src, int layout,
+    int packed_ld, const _Float16* __restrict__ attr_mask, _Float16* __restrict__ dst, const int32_t* __restrict__ seq_start,
+    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, float scaler) {
+#if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
+  using T = _Float16;
+  constexpr int NKT = kSplitHalfTiles;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  unsigned char* kv = smem_raw;
+  int* tok_of_pos = reinterpret_cast<int*>(smem_raw + kWideKvBytes);
+  float* red = reinterpret_cast<float*>(smem_raw + kWideKvBytes + kSplitKeys * sizeof(int));   // [2][4 tiles][2 halves][16]
+
+  const int b = min(max(seq_start[batch + 1 + blockIdx.z], 0), batch - 1), head = blockIdx.y, qblock = blockIdx.x;
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  const int len = t1 - t0;
+  if (len <= 0) return;
+  const int H = heads * kD;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int tile_w = wave & 3, half = wave >> 2;
+  const int l16 = lane & 15, g = lane >> 4;
+  const int kt_base = half * NKT;                            // first key tile of this half
+
+  const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
+  const int n_tiles = last_pos / 16 + 1;                     // 16-row tiles that hold at least one token
+  if (qblock * 4 >= n_tiles) return;                         // no token among this workgroup's queries
+  for (int i = threadIdx.x; i < kSplitKeys; i += kSplitThreads) tok_of_pos[i] = -1;
+  __syncthreads();
+  for (int tt = threadIdx.x; tt < len; tt += kSplitThreads) {
+    const int pos = word_idx[t0 + tt];
+    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = tt;     // relative to the sequence's first packed row
+  }
+  __syncthreads();
+
+  // Rows come in whole groups of four key tiles (what a step of the QK loop reads).  One DMA instruction fills eight
+  // slots; lane -> slot 8 i + lane / 8, 16-byte chunk (lane & 7) ^ swizzle.
+  const int rows_in = min((n_tiles + 3) / 4 * 64, kSplitKeys);
+  auto stage = [&](const T* __restrict__ src) {
+    const T* base = layout == 1 ? src + (size_t)t0 * packed_ld + head * kD : src + ((size_t)b * heads + head) * seq_len * kD;
+    const uint32_t bytes = layout == 1 ? ((uint32_t)(len - 1) * (uint32_t)packed_ld + kD) * 2u : (uint32_t)seq_len * kD * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, (int)bytes, 0x00020000);
+    for (int i = wave; i < rows_in / 8; i += kSplitThreads / kWave) {
+      const int slot = i * 8 + (lane >> 3);
+      const int key = wide_slot(slot);
+      const int c = (lane & 7) ^ wide_swizzle(slot);
+      const int tk = tok_of_pos[key];
+      const uint32_t row_off = layout == 1 ? (uint32_t)tk * (uint32_t)packed_ld : (uint32_t)key * kD;
+      const uint32_t voff = tk >= 0 ? (row_off + (uint32_t)c * 8u) * 2u : 0x80000000u;      // out of range: zeros
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, ET_ATTN_LDS_PTR(kv + i * 1024), 16, voff, 0, 0, 0);
+    }
+  };
+  stage(k_src);
+
+  const int qt = qblock * 4 + tile_w;                        // this wavefront's 16-query tile
+  const bool active = qt < n_tiles;                          // wave-uniform
+  const int q = qt * 16 + l16;
+  const int tq = (active && q < kSplitKeys) ? tok_of_pos[q] : -1;
+  const T* mrow = attr_mask + ((size_t)b * seq_len + min(q, seq_len - 1)) * seq_len;
+  const bool vec_mask = (seq_len & 7) == 0;                  // mask rows start at multiples of 16 bytes
+  auto q_off = [&](int tk, int pos) -> size_t {
+    return layout == 1 ? (size_t)(t0 + tk) * packed_ld + head * kD : (((size_t)b * heads + head) * seq_len + pos) * kD;
+  };
+
+  // Q operand of this lane (zeros for a query position without a token: its result is never stored)
+  half8 bqh[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bqh[ks][j] = (_Float16)0;
+    if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + q_off(tq, q) + ks * 32 + g * 8);
+  }
+
+  // ---- the additive bias of this half of the mask row: all loads of the row in flight before the first use -------
+  float s[NKT][4];                                           // s[2 P], s[2 P + 1]: keys base + 8 g + 0..3, + 4..7 of pair P
+  {
+    int g8 = g * 8;
+    asm volatile("" : "+v"(g8));       // opaque: the clamped offsets are recomputed, not kept in registers
+    if (vec_mask) {
+      half8 m8[NKT / 2];
+#pragma unroll
+      for (int kp = 0; kp < NKT / 2; ++kp)
+        m8[kp] = *reinterpret_cast<const half8*>(mrow + min((kt_base + 2 * kp) * 16 + g8, seq_len - 8));
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kp = 0; kp < NKT / 2; ++kp) {
+        const int key0 = (kt_base + 2 * kp) * 16 + g8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? (1.0f - (float)m8[kp][j]) * -10000.0f : -INFINITY;
+      }
+    } else {
+#pragma unroll
+      for (int kp = 0; kp < NKT / 2; ++kp) {
+        const int key0 = (kt_base + 2 * kp) * 16 + g8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const T m = mrow[min(key0 + j, seq_len - 1)];
+          s[2 * kp + (j >> 2)][j & 3] = key0 + j < seq_len ? (1.0f - (float)m) * -10000.0f : -INFINITY;
+        }
+        if (kp % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+
+  wide_wait_dma();
+  __syncthreads();                                           // K is in place
+
+  // ---- S^T = K Q^T, four key tiles at a time -----------------------------------------------------------------------
+  if (active) {
+#pragma unroll
+    for (int kg = 0; kg < NKT / 4; ++kg) {
+      if (kt_base + kg * 4 < n_tiles) {                      // wave-uniform; the rows of a started group are all staged
+        half8 a[4][2];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          // row l16 of tile t of the group: pair t >> 1, first or second tile t & 1
+          const int slot = wide_slot((kt_base + kg * 4 + (t & ~1)) * 16 + (l16 >> 2) * 8 + (t & 1) * 4 + (l16 & 3));
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks)
+            a[t][ks] = *reinterpret_cast<const half8*>(kv + slot * 128 + (((ks * 4 + g) ^ wide_swizzle(slot)) * 16));
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][ks], bqh[ks], acc, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float sc = h2f(f2h(acc[r]));                 // the score is stored in half
+            s[kg * 4 + t][r] = sc * scaler + s[kg * 4 + t][r];
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();                                           // every wavefront has read K for the last time
+  stage(v_src);                                              // arrives while the softmax runs
+
+  // ---- masked softmax: each half over its registers, maxima and sums exchanged through LDS --------------------
+  float* red_max = red;
+  float* red_sum = red + 4 * 2 * 16;
+  {
+    float mx = seq_len < kSplitKeys ? 0.f : -INFINITY;       // the clamp at 0 holds below 1024 keys
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][r]);
+    mx = xor_lanes_16_32_max(mx);
+    if (g == 0) red_max[(tile_w * 2 + half) * 16 + l16] = mx;
+  }
+  wide_wait_lds();
+  wide_barrier();
+  {
+    const float mx = fmaxf(red_max[(tile_w * 2) * 16 + l16], red_max[(tile_w * 2 + 1) * 16 + l16]) * kLog2e;
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[kt][r] = __builtin_amdgcn_exp2f(s[kt][r] * kLog2e - mx);
+        sum += s[kt][r];
+      }
+    sum = xor_lanes_16_32_sum(sum);
+    if (g == 0) red_sum[(tile_w * 2 + half) * 16 + l16] = sum;
+  }
+  wide_wait_lds();
+  wide_barrier();
+  {
+    const float sum = red_sum[(tile_w * 2) * 16 + l16] + red_sum[(tile_w * 2 + 1) * 16 + l16] + 1e-6f;
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[kt][r] *= inv;
+  }
+  wide_wait_dma();
+  __syncthreads();                                           // V is in place
+
+  // ---- O^T = V^T P^T, each half over its keys, two key tiles (one MFMA k range) at a time ------------------------
+  float4v o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+  if (active) {
+#pragma unroll
+    for (int kp = 0; kp < NKT / 2; ++kp) {
+      if (kt_base + 2 * kp < n_tiles) {                      // wave-uniform
+        half8 p;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[r] = f2h(s[2 * kp][r]);
+          p[4 + r] = f2h(s[2 * kp + 1][r]);
+        }
+        typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u2 raw[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          const int slot = wide_slot((kt_base + 2 * kp) * 16 + g * 8 + kk);
+          raw[kk] = *reinterpret_cast<const u2*>(kv + slot * 128 + (((l16 >> 1) ^ wide_swizzle(slot)) * 16) + (l16 & 1) * 8);
+        }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          u4 lo, hi;
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            lo[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x05040100u);
+            hi[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x07060302u);
+          }
+          o[2 * jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, lo), p, o[2 * jj], 0, 0, 0);
+          o[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, hi), p, o[2 * jj + 1], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- the second half hands its part of O over (through the K/V rows, free now), the first adds and stores ------
+  __syncthreads();
+  float4v* xo = reinterpret_cast<float4v*>(smem_raw);        // [4 tiles][64 lanes][4]
+  if (half == 1) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) xo[(tile_w * kWave + lane) * 4 + dt] = o[dt];
+  }
+  __syncthreads();
+  if (half == 0 && tq >= 0) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      const float4v other = xo[(tile_w * kWave + lane) * 4 + dt];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] += other[r];
+    }
+    half8 v0, v1;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v0[4 * r + j] = f2h(o[j][r]);
+        v1[4 * r + j] = f2h(o[j][2 + r]);
+      }
+    T* orow = dst + (size_t)(t0 + tq) * H + head * kD + g * 16;
+    *reinterpret_cast<half8*>(orow) = v0;
+    *reinterpret_cast<half8*>(orow + 8) = v1;
+  }
+#endif
+}
+
 template <typename T>
 void attention_split_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                             void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                             float scaler, hipStream_t stream) {
   const size_t smem = 2 * LongSmem<T>::kTileBytes + (size_t)kSplitKeys * sizeof(int) + 2 * 4 * 2 * 16 * sizeof(float);
+  dim3 grid(kSplitKeys / 64, heads, batch);
+  if constexpr (sizeof(T) == 2) {
+    allow_dynamic_lds(reinterpret_cast<const void*>(attention_wide_kernel), kWideSmem);
+    attention_wide_kernel<<<grid, kSplitThreads, kWideSmem, stream>>>(
+        (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, layout, packed_ld, (const _Float16*)attr_mask,
+        (_Float16*)dst, seq_start, word_idx, batch, seq_len, heads, scaler);
+    return;
+  }
   auto kern = attention_split_kernel<T>;
   allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem);
-  dim3 grid(kSplitKeys / 64, heads, batch);
   kern<<<grid, kSplitThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
                                               (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch, seq_len, heads,
                                               scaler);

@@ -308,7 +308,7 @@ def test_fused_attention_with_resident_keys(k, B, heads, S, holes, weird):
 @pytest.mark.parametrize("S,d,holes,weird", [(40, 32, False, False), (70, 128, True, True), (33, 8, True, False),
                                              (16, 256, False, True), (600, 64, False, False), (513, 64, True, True),
                                              (1024, 64, False, True), (1000, 32, True, False),
-                                             (1023, 64, True, False), (768, 64, False, True)])
+                                             (1023, 64, True, False), (768, 64, False, True), (900, 64, True, True)])
 def test_fused_attention_other_head_sizes_and_long_sequences(k, dtype, S, d, holes, weird):
     """size_per_head other than 64 (the reference op takes any, tf_op/bert_transformer_op.cc:53-57) and 512 < seq_len <= 1024
     (its softmax launcher's last branch, cuda/attention.cu:345-356; no clamp of the maximum at 1024 keys)."""
