@@ -1738,7 +1738,7 @@ void attention_split_launch(const void* q, const void* k, const void* v, int lay
                             void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                             float scaler, hipStream_t stream) {
   const size_t smem = 2 * LongSmem<T>::kTileBytes + (size_t)kSplitKeys * sizeof(int) + 2 * 4 * 2 * 16 * sizeof(float);
-  dim3 grid(kSplitKeys / 64, heads, batch);
+  dim3 grid((seq_len + 63) / 64, heads, batch);              // blocks of 64 queries that can hold a token
   if constexpr (sizeof(T) == 2) {
     allow_dynamic_lds(reinterpret_cast<const void*>(attention_wide_kernel), kWideSmem);
     attention_wide_kernel<<<grid, kSplitThreads, kWideSmem, stream>>>(
