@@ -273,8 +273,8 @@ et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, 
  *   qkv_layout 1: q/k/v point into packed token-major rows (row t, column head*d + j) with row
  *                 stride `packed_ld` elements (bias already added).
  *   dst packed [T,heads*d].  workspace: et_seq_workspace_bytes(B).
- * seq_len <= 1024; size_per_head <= 256 with head rows of whole 16-byte pieces.  size_per_head = 64 with
- * seq_len <= 512 runs the MFMA kernels, every other shape a slower general kernel with the same arithmetic. */
+ * seq_len <= 1024; size_per_head <= 256 with head rows of whole 16-byte pieces.  size_per_head = 64 runs the
+ * MFMA kernels, every other head size a slower general kernel with the same arithmetic. */
 et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v, int qkv_layout,
                        int packed_ld, const void* attr_mask, void* dst,
                        const int32_t* valid_word_num_dev, int batch_size, int seq_len,
