@@ -828,7 +828,7 @@ void attention_long_launch(const void* q, const void* k, const void* v, int layo
                            float scaler, hipStream_t stream) {
   const size_t smem = LongSmem<T>::kTileBytes + (size_t)NKT * 16 * sizeof(int);
   auto kern = attention_long_kernel<T, NKT>;
-  dim3 grid(NKT / 4, heads, batch);
+  dim3 grid((seq_len + 63) / 64, heads, batch);               // blocks of 64 queries that can hold a token
   kern<<<grid, kAttnThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld, (const T*)attr_mask,
                                              (T*)dst, seq_start, word_idx, batch, seq_len, heads, scaler);
 }
