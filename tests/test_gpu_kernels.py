@@ -338,6 +338,44 @@ def test_fused_attention_other_head_sizes_and_long_sequences(k, dtype, S, d, hol
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("S", [300, 712])
+def test_fused_attention_long_sequences_same_bits_in_any_batch(k, dtype, S):
+    """A sequence's attention output does not depend on what else is in the batch or where it stands in it: the same
+    five sequences in two orders, and one of them alone, give the same bits (kernels that split a sequence's queries
+    or keys over workgroups and wavefronts: keys resident in LDS up to 512 positions, key halves beyond)."""
+    print("attention batch independence", dtype, S, flush=True)
+    heads, d = 3, 64
+    H = heads * d
+    rng = np.random.RandomState(S)
+    lens = [S, 1, S // 2 + 3, 17, S - 9]
+    rows = [o.rnd(rng.randn(n, 3 * H), dtype) for n in lens]
+    attr_seq = [o.rnd((rng.random_sample((S, S)) < 0.8).astype(np.float32), dtype) for _ in lens]
+
+    def run(order):
+        B = len(order)
+        mask = np.zeros((B, S), np.int32)
+        for i, j in enumerate(order):
+            mask[i, :lens[j]] = 1
+        _, T, bi, wi, _ = o.input_op_fast(np.zeros((B, S, 1), np.float32), mask)
+        packed = np.zeros((B * S, 3 * H), o._np_dtype(dtype))
+        packed[:T] = np.concatenate([rows[j] for j in order])
+        attr = np.stack([attr_seq[j] for j in order])
+        p = dict(B=B, S=S, T=T, bi=bi, wi=wi)
+        bi_d, wi_d, vwn = _idx_dev(p)
+        pk = dev(packed)
+        out = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(attr), vwn, B, S, heads, d, bi_d, wi_d).cpu().numpy()
+        starts = np.concatenate([[0], np.cumsum([lens[j] for j in order])])
+        return {j: out[starts[i]:starts[i + 1]] for i, j in enumerate(order)}
+
+    a = run([0, 1, 2, 3, 4])
+    b = run([3, 4, 0, 2, 1])
+    c = run([2])
+    for j in range(5):
+        assert np.array_equal(a[j], b[j]), j
+    assert np.array_equal(a[2], c[2])
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 def test_fused_attention_many_sequences_head_groups(k, dtype):
     """A batch large enough that one workgroup serves a group of 4 heads (shared mask registers, positions and
     zero fill across heads, next head prefetched): holes in the mask, an attention mask unrelated to it."""
