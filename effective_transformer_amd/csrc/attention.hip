@@ -948,31 +948,25 @@ void attention_resident_kernel(
       if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + src_off(tq, q) + ks * 32 + g * 8);
     }
 
-    // ---- the additive bias of the mask row first: no branch between its loads, eight in flight ------------------
+    // ---- the additive bias of the mask row first ------------------------------------------------------------------
     float s[NKT][4];
     const int n_groups = (n_tiles + 3) / 4;
     // (opaque to the compiler, or it would keep the clamped offsets of all key tiles in registers across query tiles)
     int g4 = g * 4;
     asm volatile("" : "+v"(g4));
     // (1 - m) * -10000 as one fma: 1 - m is exact in float for a half m, so both forms round the same real number once
-    if (seq_len == kSp) {
-      // every key of every tile exists
+    if (vec_mask) {
+      // all loads of the row in flight before the first conversion: one memory latency per query tile
+      mask4 m4[NKT];
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) {
-        const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + kt * 16 + g4);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s[kt][r] = __builtin_fmaf((float)m4[r], 10000.0f, -10000.0f);
-        if (kt % 8 == 7) __builtin_amdgcn_sched_barrier(0);
-      }
-    } else if (vec_mask) {
+      for (int kt = 0; kt < NKT; ++kt) m4[kt] = *reinterpret_cast<const mask4*>(mrow + min(kt * 16 + g4, seq_len - 4));
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt) {
         const int key0 = kt * 16 + g4;
-        const mask4 m4 = *reinterpret_cast<const mask4*>(mrow + min(key0, seq_len - 4));
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          s[kt][r] = key0 < seq_len ? __builtin_fmaf((float)m4[r], 10000.0f, -10000.0f) : -INFINITY;
-        if (kt % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+          s[kt][r] = key0 < seq_len ? __builtin_fmaf((float)m4[kt][r], 10000.0f, -10000.0f) : -INFINITY;
       }
     } else {
 #pragma unroll
