@@ -834,22 +834,40 @@ void attention_long_launch(const void* q, const void* k, const void* v, int layo
 }
 
 // ------------------------------------------------------------------------------------------
+// K / V rows brought into LDS by DMA (the resident-key kernels below): rows of 128 bytes without padding, one
+// `buffer_load ... lds` instruction fills eight of them (lane -> row lane / 8, 16-byte chunk lane & 7).  A row without
+// a token is requested beyond its buffer descriptor's range and arrives as zeros.
+// Which key a row of an MFMA tile stands for is free as long as K, the mask and V agree: row m of the first tile of a
+// pair (32 keys from `base`) is key base + (m >> 2) * 8 + (m & 3), of the second tile 4 keys further.  A lane's scores
+// of a pair are then 8 consecutive keys: one 16-byte load of its mask row, and the P operand of the P.V MFMA is in
+// natural key order.  Key row `key` lies in slot key ^ ((key >> 3) & 1) (the two rows of a half-wave of the 8-byte V
+// reads, 8 keys apart, land on different halves of the banks), and the 16-byte chunks of a slot are XOR-swizzled with
+// slot bits 1, 3 and 4 (the 16 rows x one chunk of a K operand read cover all 64 banks).
+// ------------------------------------------------------------------------------------------
+#define ET_ATTN_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+__device__ __forceinline__ int wide_slot(int key) { return key ^ ((key >> 3) & 1); }
+__device__ __forceinline__ int wide_swizzle(int slot) { return ((slot >> 1) & 1) | ((slot >> 2) & 6); }
+// s_waitcnt immediates of gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+__device__ __forceinline__ void wide_wait_dma() { __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8) | (0 << 14)); }
+__device__ __forceinline__ void wide_wait_lds() { __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14)); }
+// barrier without the fence of __syncthreads(), which would wait for every DMA in flight
+__device__ __forceinline__ void wide_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// ------------------------------------------------------------------------------------------
 // fp16 fused attention for 128 < seq_len <= 512 with K and V of the whole sequence resident in LDS: one workgroup of
-// 8 wavefronts per (head, sequence) (or per share of its query tiles, see `qsplit`).  K and V are staged once (73 + 81
-// KB at 512 keys) instead of once per block of 64 queries, and after that one barrier the wavefronts run their
-// 16-query tiles independently: S^T = K Q^T over all key tiles, the softmax over the registers, O^T = V^T P^T.  The
-// arithmetic, its order and the rounding points are those of attention_long_kernel (the results are the same bits).
+// 8 wavefronts per (head, sequence) (or per share of its query tiles, see `qsplit`).  K and V arrive once by DMA (64 +
+// 64 KB at 512 keys, all requests in flight at once, layout above) instead of once per block of 64 queries, and after
+// that one barrier the wavefronts run their 16-query tiles independently: S^T = K Q^T over all key tiles, the softmax
+// over the registers, O^T = V^T P^T.  Arithmetic and rounding points per element are those of attention_long_kernel.
 // ------------------------------------------------------------------------------------------
 constexpr int kResThreads = 512;
-constexpr int kResWaves = kResThreads / kWave;
+[[maybe_unused]] constexpr int kResWaves = kResThreads / kWave;
 
 template <int NKT>
 struct ResSmem {
   static constexpr int kSp = NKT * 16;
-  static constexpr int kQS = AttnCfg<_Float16>::kQkStride;
-  static constexpr int kVR = AttnCfg<_Float16>::kVStride;
-  static constexpr size_t kKBytes = (size_t)kSp * kQS * 2;
-  static constexpr size_t kVBytes = (size_t)kSp * kVR * 2;
+  static constexpr size_t kKBytes = (size_t)kSp * 128;
+  static constexpr size_t kVBytes = (size_t)kSp * 128;
   static constexpr size_t kBytes = kKBytes + kVBytes + (size_t)kSp * sizeof(int);
 };
 
@@ -860,17 +878,14 @@ void attention_resident_kernel(
     int packed_ld, const _Float16* __restrict__ attr_mask, _Float16* __restrict__ dst,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads,
     int qsplit, float scaler) {
+#if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   using T = _Float16;
   using Sm = ResSmem<NKT>;
-  using C = Chunk16<T>;
-  using V16 = typename C::vec;
-  constexpr int kQS = Sm::kQS, kVR = Sm::kVR, kSp = Sm::kSp;
-  constexpr int kCpr = kD / C::kElems;                       // 16-byte pieces per head row
-  typedef T mask4 __attribute__((ext_vector_type(4)));
+  constexpr int kSp = Sm::kSp;
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* Ks = reinterpret_cast<T*>(smem_raw);
-  T* Vs = reinterpret_cast<T*>(smem_raw + Sm::kKBytes);
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  unsigned char* ks = smem_raw;
+  unsigned char* vs = smem_raw + Sm::kKBytes;
   int* tok_of_pos = reinterpret_cast<int*>(smem_raw + Sm::kKBytes + Sm::kVBytes);
 
   const int b = min(max(seq_start[batch + 1 + blockIdx.y], 0), batch - 1);
@@ -880,7 +895,7 @@ void attention_resident_kernel(
   if (len <= 0) return;
   const int H = heads * kD;
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int l16 = lane & 15, g = lane >> 4;
 
   const int last_pos = min(max(word_idx[t1 - 1], 0), seq_len - 1);
@@ -890,51 +905,55 @@ void attention_resident_kernel(
   __syncthreads();
   for (int tt = threadIdx.x; tt < len; tt += kResThreads) {
     const int pos = word_idx[t0 + tt];
-    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = t0 + tt;
+    if (pos >= 0 && pos < seq_len) tok_of_pos[pos] = tt;     // relative to the sequence's first packed row
   }
   __syncthreads();
 
-  auto src_off = [&](int t, int pos) -> size_t {
-    return layout == 1 ? (size_t)t * packed_ld + head * kD : (((size_t)b * heads + head) * seq_len + pos) * kD;
-  };
-  // K and V rows of every group of four key tiles that holds a token (the loops below run over such groups), zeros
-  // where no token sits; four pieces of each per thread in flight
+  // K and V rows of every group of four key tiles that holds a token (the loops below run over such groups)
+  const int n_groups = (n_tiles + 3) / 4;
   {
-    const int rows = min(kSp, ((n_tiles + 3) / 4) * 64);
-    const int pieces = rows * kCpr;
-    constexpr int kFly = 4;
-    for (int i0 = threadIdx.x; i0 < pieces; i0 += kFly * kResThreads) {
-      V16 rk[kFly], rv[kFly];
-#pragma unroll
-      for (int u = 0; u < kFly; ++u) {
-        const int i = i0 + u * kResThreads;
-        const int row = i / kCpr, c = i - row * kCpr;
-#pragma unroll
-        for (int j = 0; j < C::kElems; ++j) {
-          rk[u][j] = (T)0;
-          rv[u][j] = (T)0;
-        }
-        const int tk = i < pieces ? tok_of_pos[row] : -1;
-        if (tk >= 0) {
-          const size_t off = src_off(tk, row) + c * C::kElems;
-          rk[u] = *reinterpret_cast<const V16*>(k_src + off);
-          rv[u] = *reinterpret_cast<const V16*>(v_src + off);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kFly; ++u) {
-        const int i = i0 + u * kResThreads;
-        if (i < pieces) {
-          const int row = i / kCpr, c = i - row * kCpr;
-          *reinterpret_cast<V16*>(Ks + row * kQS + c * C::kElems) = rk[u];
-          *reinterpret_cast<V16*>(Vs + row * kVR + c * C::kElems) = rv[u];
-        }
-      }
+    const int rows_in = min(kSp, n_groups * 64);
+    const T* kbase = layout == 1 ? k_src + (size_t)t0 * packed_ld + head * kD : k_src + ((size_t)b * heads + head) * seq_len * kD;
+    const T* vbase = layout == 1 ? v_src + (size_t)t0 * packed_ld + head * kD : v_src + ((size_t)b * heads + head) * seq_len * kD;
+    const uint32_t bytes = layout == 1 ? ((uint32_t)(len - 1) * (uint32_t)packed_ld + kD) * 2u : (uint32_t)seq_len * kD * 2u;
+    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kbase), 0, (int)bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vbase), 0, (int)bytes, 0x00020000);
+    for (int i = wave; i < rows_in / 8; i += kResWaves) {
+      const int slot = i * 8 + (lane >> 3);
+      const int key = wide_slot(slot);
+      const int c = (lane & 7) ^ wide_swizzle(slot);
+      const int tk = tok_of_pos[key];
+      const uint32_t row_off = layout == 1 ? (uint32_t)tk * (uint32_t)packed_ld : (uint32_t)key * kD;
+      const uint32_t voff = tk >= 0 ? (row_off + (uint32_t)c * 8u) * 2u : 0x80000000u;      // out of range: zeros
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, ET_ATTN_LDS_PTR(ks + i * 1024), 16, voff, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, ET_ATTN_LDS_PTR(vs + i * 1024), 16, voff, 0, 0, 0);
     }
   }
+  wide_wait_dma();
   __syncthreads();
 
-  const bool vec_mask = (seq_len & 3) == 0;
+  // Operand addresses: a lane-dependent base plus a compile-time offset per tile.  The slot flip touches bit 0 of the
+  // row and the swizzle bits 1, 3, 4, none of which the tile's part of the row number (multiples of 32, +4 for the
+  // second tile of a pair) reaches, so both are constants of the lane.
+  //   K, row l16 of a tile: key row L = (l16 >> 2) * 8 + (l16 & 3) within the pair, chunk ks * 4 + g
+  const unsigned char* kbase_ks[2];
+  {
+    const int L = wide_slot((l16 >> 2) * 8 + (l16 & 3));
+    const int sw = wide_swizzle(L);
+#pragma unroll
+    for (int ks2 = 0; ks2 < 2; ++ks2) kbase_ks[ks2] = ks + L * 128 + (((ks2 * 4 + g) ^ sw) * 16);
+  }
+  //   V, key g * 8 + kk of a pair (kk = 4 a + 2 b + c), features 4 l16 ..: base by (b, c), offset 512 a
+  const unsigned char* vbase_bc[2][2];
+#pragma unroll
+  for (int bb = 0; bb < 2; ++bb)
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const int slot = wide_slot(g * 8 + 2 * bb + cc);
+      vbase_bc[bb][cc] = vs + slot * 128 + (((l16 >> 1) ^ wide_swizzle(slot)) * 16) + (l16 & 1) * 8;
+    }
+
+  const bool vec_mask = (seq_len & 7) == 0;                  // mask rows start at multiples of 16 bytes
   for (int qt = part + qsplit * wave; qt < n_tiles; qt += qsplit * kResWaves) {
     const int q = qt * 16 + l16;
     const int tq = tok_of_pos[q];
@@ -942,42 +961,44 @@ void attention_resident_kernel(
     // Q operand of this lane (zeros for a query position without a token: its result is never stored)
     half8 bqh[2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks2 = 0; ks2 < 2; ++ks2) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) bqh[ks][j] = (_Float16)0;
-      if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + src_off(tq, q) + ks * 32 + g * 8);
+      for (int j = 0; j < 8; ++j) bqh[ks2][j] = (_Float16)0;
+      if (tq >= 0) {
+        const size_t qo = layout == 1 ? (size_t)(t0 + tq) * packed_ld + head * kD
+                                      : (((size_t)b * heads + head) * seq_len + q) * kD;
+        bqh[ks2] = *reinterpret_cast<const half8*>(q_src + qo + ks2 * 32 + g * 8);
+      }
     }
 
-    // ---- the additive bias of the mask row first ------------------------------------------------------------------
-    float s[NKT][4];
-    const int n_groups = (n_tiles + 3) / 4;
-    // (opaque to the compiler, or it would keep the clamped offsets of all key tiles in registers across query tiles)
-    int g4 = g * 4;
-    asm volatile("" : "+v"(g4));
+    // ---- the additive bias of the mask row first: the whole row requested before any of it is converted --------
+    float s[NKT][4];                                         // s[2 P], s[2 P + 1]: keys 32 P + 8 g + 0..3, + 4..7
+    // (opaque to the compiler, or it would keep the clamped offsets of all pairs in registers across query tiles)
+    int g8 = g * 8;
+    asm volatile("" : "+v"(g8));
     // (1 - m) * -10000 as one fma: 1 - m is exact in float for a half m, so both forms round the same real number once
     if (vec_mask) {
-      // all loads of the row in flight before the first conversion: one memory latency per query tile
-      mask4 m4[NKT];
+      half8 m8[NKT / 2];
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) m4[kt] = *reinterpret_cast<const mask4*>(mrow + min(kt * 16 + g4, seq_len - 4));
+      for (int kp = 0; kp < NKT / 2; ++kp) m8[kp] = *reinterpret_cast<const half8*>(mrow + min(kp * 32 + g8, seq_len - 8));
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) {
-        const int key0 = kt * 16 + g4;
+      for (int kp = 0; kp < NKT / 2; ++kp) {
+        const int key0 = kp * 32 + g8;
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          s[kt][r] = key0 < seq_len ? __builtin_fmaf((float)m4[kt][r], 10000.0f, -10000.0f) : -INFINITY;
+        for (int j = 0; j < 8; ++j)
+          s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? __builtin_fmaf((float)m8[kp][j], 10000.0f, -10000.0f) : -INFINITY;
       }
     } else {
 #pragma unroll
-      for (int kt = 0; kt < NKT; ++kt) {
-        const int key0 = kt * 16 + g4;
+      for (int kp = 0; kp < NKT / 2; ++kp) {
+        const int key0 = kp * 32 + g8;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const T m = mrow[min(key0 + r, seq_len - 1)];
-          s[kt][r] = key0 + r < seq_len ? __builtin_fmaf((float)m, 10000.0f, -10000.0f) : -INFINITY;
+        for (int j = 0; j < 8; ++j) {
+          const T m = mrow[min(key0 + j, seq_len - 1)];
+          s[2 * kp + (j >> 2)][j & 3] = key0 + j < seq_len ? __builtin_fmaf((float)m, 10000.0f, -10000.0f) : -INFINITY;
         }
-        if (kt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+        if (kp % 2 == 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
     // ---- S^T = K Q^T, four key tiles at a time (rows without a token are zero: score 0) ---------------------
@@ -987,11 +1008,12 @@ void attention_resident_kernel(
 #pragma unroll
         for (int kc = 0; kc < 4; ++kc) {
           const int kt = kg * 4 + kc;
+          // row l16 of tile kt: pair kt >> 1, first or second tile kt & 1 (4 rows further)
           float4v acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int ks = 0; ks < 2; ++ks) {
-            const half8 a = *reinterpret_cast<const half8*>(Ks + (kt * 16 + l16) * kQS + ks * 32 + g * 8);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bqh[ks], acc, 0, 0, 0);
+          for (int ks2 = 0; ks2 < 2; ++ks2) {
+            const half8 a = *reinterpret_cast<const half8*>(kbase_ks[ks2] + ((kt & ~1) * 16 + (kt & 1) * 4) * 128);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bqh[ks2], acc, 0, 0, 0);
           }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
@@ -1045,8 +1067,7 @@ void attention_resident_kernel(
         u2 raw[8];
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-          const int key = kp * 32 + (kk >> 2) * 16 + g * 4 + (kk & 3);
-          raw[kk] = *reinterpret_cast<const u2*>(Vs + key * kVR + l16 * 4);
+          raw[kk] = *reinterpret_cast<const u2*>(vbase_bc[(kk >> 1) & 1][kk & 1] + (kp * 32 + (kk & 4)) * 128);
         }
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
@@ -1071,11 +1092,12 @@ void attention_resident_kernel(
           v0[4 * r + j] = f2h(o[j][r]);
           v1[4 * r + j] = f2h(o[j][2 + r]);
         }
-      T* orow = dst + (size_t)tq * H + head * kD + g * 16;
+      T* orow = dst + (size_t)(t0 + tq) * H + head * kD + g * 16;
       *reinterpret_cast<half8*>(orow) = v0;
       *reinterpret_cast<half8*>(orow + 8) = v1;
     }
   }
+#endif
 }
 
 inline int attention_cu_count() {
@@ -1462,24 +1484,11 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
 // bytes) arrives by DMA, all requests in flight together with the mask row and Q, instead of chunk after chunk through
 // registers with a fetch latency each; V follows into the same rows while the softmax runs.  A row without a token is
 // requested beyond its buffer descriptor's range and arrives as zeros.
-// Which key a row of an MFMA tile stands for is free as long as K, the mask and V agree: row m of the first tile of a
-// pair (32 keys from `base`) is key base + (m >> 2) * 8 + (m & 3), of the second tile 4 keys further.  A lane's scores
-// of a pair are then 8 consecutive keys: one 16-byte load of its mask row, and the P operand of the P.V MFMA is in
-// natural key order.  Key row `key` lies in slot key ^ ((key >> 3) & 1) (the two rows of a half-wave of the 8-byte V
-// reads, 8 keys apart, land on different halves of the banks), and the 16-byte chunks of a slot are XOR-swizzled with
-// slot bits 1, 3 and 4 (the 16 rows x one chunk of a K operand read cover all 64 banks).  Arithmetic and rounding
-// points per element are those of the split kernel.
+// Rows, key order and swizzle as described above the resident-key kernel.  Arithmetic and rounding points per element
+// are those of the split kernel.
 // ------------------------------------------------------------------------------------------
 constexpr int kWideKvBytes = kSplitKeys * 128;
 constexpr int kWideSmem = kWideKvBytes + kSplitKeys * (int)sizeof(int) + 2 * 4 * 2 * 16 * (int)sizeof(float);
-#define ET_ATTN_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-__device__ __forceinline__ int wide_slot(int key) { return key ^ ((key >> 3) & 1); }
-__device__ __forceinline__ int wide_swizzle(int slot) { return ((slot >> 1) & 1) | ((slot >> 2) & 6); }
-// s_waitcnt immediates of gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
-__device__ __forceinline__ void wide_wait_dma() { __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8) | (0 << 14)); }
-__device__ __forceinline__ void wide_wait_lds() { __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14)); }
-// barrier without the fence of __syncthreads(), which would wait for every DMA in flight
-__device__ __forceinline__ void wide_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
     const _Float16* __restrict__ q_src, const _Float16* __restrict__ k_src, const _Float16* __restrict__ v_src, int layout,
