@@ -84,3 +84,26 @@ def test_sweep_prints_one_row_per_published_row(capsys):
         assert cells[5] == "%.2f (Readme.md:%d)" % (published, line)
         ms, T = float(cells[6]), int(cells[4])
         assert ms > 0 and abs(float(cells[8]) - T / ms * 1e3) <= 0.01 * T / ms * 1e3
+
+
+def test_sweep_long_rows_stay_within_the_reach_of_the_reference():
+    """The second table's rows: precisions of the reference, max_seq up to the 1024 positions its softmax launch
+    covers (cuda/attention.cu:345-356), and the benchmark's length recipe needs 2 * avg - max >= 1."""
+    assert sweep.build_parser().parse_args(["--long", "--max-seq", "256"]).long
+    for precision, max_seq, avg_seq, batch in sweep.LONG_ROWS:
+        assert precision in ("fp16", "fp32") and 64 < max_seq <= 1024 and batch >= 1
+        assert 2 * avg_seq - max_seq >= 1 and avg_seq <= max_seq
+
+
+@pytest.mark.gpu
+def test_sweep_long_prints_its_rows(capsys):
+    print("sample sweep --long", flush=True)
+    args = sweep.build_parser().parse_args(["--long", "--iters", "2", "--precision", "fp16", "--max-seq", "256"])
+    capsys.readouterr()
+    sweep.main_long(args)
+    rows = [l for l in capsys.readouterr().out.splitlines() if l.startswith("| fp16")]
+    assert [r.split("|")[2].strip() for r in rows] == ["128", "256"]
+    for row in rows:
+        cells = [c.strip() for c in row.strip("|").split("|")]
+        ms, std, T = float(cells[5]), float(cells[6]), int(cells[4])
+        assert ms > 0 and std > 0 and abs(float(cells[8]) - T / ms * 1e3) <= 0.01 * T / ms * 1e3
