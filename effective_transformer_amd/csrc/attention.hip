@@ -1595,6 +1595,22 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
     }
   }
 
+  // operand addresses: a lane-dependent base (this half's first row included) plus a compile-time offset per tile
+  const unsigned char* kbase_ks[2];
+  const unsigned char* vbase_bc[2][2];
+  {
+    const int L = wide_slot((l16 >> 2) * 8 + (l16 & 3));
+    const int sw = wide_swizzle(L);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) kbase_ks[ks] = kv + (kt_base * 16 + L) * 128 + (((ks * 4 + g) ^ sw) * 16);
+#pragma unroll
+    for (int bb = 0; bb < 2; ++bb)
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        const int slot = wide_slot(g * 8 + 2 * bb + cc);
+        vbase_bc[bb][cc] = kv + (kt_base * 16 + slot) * 128 + (((l16 >> 1) ^ wide_swizzle(slot)) * 16) + (l16 & 1) * 8;
+      }
+  }
   wide_wait_dma();
   __syncthreads();                                           // K is in place
 
@@ -1606,11 +1622,10 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
         half8 a[4][2];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          // row l16 of tile t of the group: pair t >> 1, first or second tile t & 1
-          const int slot = wide_slot((kt_base + kg * 4 + (t & ~1)) * 16 + (l16 >> 2) * 8 + (t & 1) * 4 + (l16 & 3));
+          // row l16 of tile t of the group: pair t >> 1, first or second tile t & 1 (4 rows further)
 #pragma unroll
           for (int ks = 0; ks < 2; ++ks)
-            a[t][ks] = *reinterpret_cast<const half8*>(kv + slot * 128 + (((ks * 4 + g) ^ wide_swizzle(slot)) * 16));
+            a[t][ks] = *reinterpret_cast<const half8*>(kbase_ks[ks] + ((kg * 4 + (t & ~1)) * 16 + (t & 1) * 4) * 128);
         }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -1688,8 +1703,7 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
         u2 raw[8];
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-          const int slot = wide_slot((kt_base + 2 * kp) * 16 + g * 8 + kk);
-          raw[kk] = *reinterpret_cast<const u2*>(kv + slot * 128 + (((l16 >> 1) ^ wide_swizzle(slot)) * 16) + (l16 & 1) * 8);
+          raw[kk] = *reinterpret_cast<const u2*>(vbase_bc[(kk >> 1) & 1][kk & 1] + (kp * 32 + (kk & 4)) * 128);
         }
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
