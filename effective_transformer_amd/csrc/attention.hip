@@ -985,9 +985,14 @@ void attention_resident_kernel(
 #pragma unroll
       for (int kp = 0; kp < NKT / 2; ++kp) {
         const int key0 = kp * 32 + g8;
+        if ((kp + 1) * 32 <= seq_len) {                      // wave-uniform: every key of the pair exists
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? __builtin_fmaf((float)m8[kp][j], 10000.0f, -10000.0f) : -INFINITY;
+          for (int j = 0; j < 8; ++j) s[2 * kp + (j >> 2)][j & 3] = __builtin_fmaf((float)m8[kp][j], 10000.0f, -10000.0f);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? __builtin_fmaf((float)m8[kp][j], 10000.0f, -10000.0f) : -INFINITY;
+        }
       }
     } else {
 #pragma unroll
@@ -1577,9 +1582,14 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
 #pragma unroll
       for (int kp = 0; kp < NKT / 2; ++kp) {
         const int key0 = (kt_base + 2 * kp) * 16 + g8;
+        if ((kt_base + 2 * kp + 2) * 16 <= seq_len) {        // wave-uniform: every key of the pair exists
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? (1.0f - (float)m8[kp][j]) * -10000.0f : -INFINITY;
+          for (int j = 0; j < 8; ++j) s[2 * kp + (j >> 2)][j & 3] = (1.0f - (float)m8[kp][j]) * -10000.0f;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? (1.0f - (float)m8[kp][j]) * -10000.0f : -INFINITY;
+        }
       }
     } else {
 #pragma unroll
