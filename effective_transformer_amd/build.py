@@ -32,6 +32,12 @@ FLAGS = [
 ]
 
 
+# per source: the attention kernels keep their MFMA accumulators in VGPRs (with the accumulator registers as
+# destination every score and output value costs a v_accvgpr_read before the VALU can touch it: 24 of the 193 VALU
+# instructions per head and query tile of the short fp16 kernel)
+EXTRA_FLAGS = {"attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -41,7 +47,7 @@ def hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc(), *FLAGS, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
