@@ -189,15 +189,31 @@ struct AttnSmem {
   static constexpr size_t kBytes = 2 * kQBytes + kVtBytes + kSp * sizeof(int);
 };
 
+// Reductions over the four 16-lane rows of a wavefront (lanes l, l ^ 16, l ^ 32, l ^ 48), the result in all of them.
+// v_permlane16_swap exchanges the odd rows of its first operand with the even rows of its second, v_permlane32_swap
+// the upper half of the first with the lower half of the second: with both operands a copy of v, the two results hold
+// the two rows (halves) that have to be combined, in every lane, without a trip through the LDS crossbar.  The
+// operands of each combination are those of the xor shuffle, in one order or the other: same bits.
+// (Written as inline assembly on two float copies: with the compiler's builtin, and with integer copies handed back
+// as a vector, the second result was lost when both operands hold the same value.  The wait states in front are
+// those the compiler itself puts between a VALU write and this instruction.)
 __device__ __forceinline__ float xor_lanes_16_32_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, kWave));
-  v = fmaxf(v, __shfl_xor(v, 32, kWave));
-  return v;
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  v = fmaxf(a, b);
+  a = v;
+  b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
 }
 __device__ __forceinline__ float xor_lanes_16_32_sum(float v) {
-  v += __shfl_xor(v, 16, kWave);
-  v += __shfl_xor(v, 32, kWave);
-  return v;
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  v = a + b;
+  a = v;
+  b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return a + b;
 }
 
 // CPT = 16-byte chunks of one matrix a thread moves per head (ceil(seq rows * chunks per row / 256)).
