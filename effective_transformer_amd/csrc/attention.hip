@@ -345,6 +345,15 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
     }
   }
 
+  // where each of this lane's queries writes its output row (head 0; null without a token): the same for every head
+  T* out_row[QPW];
+#pragma unroll
+  for (int qi = 0; qi < QPW; ++qi) {
+    const int qt = wave + qi * kAttnWaves;
+    const int tq = qt < n_tiles ? tok_of_pos[qt * 16 + l16] : -1;
+    out_row[qi] = tq >= 0 ? dst + (size_t)tq * H + g * (sizeof(T) == 2 ? 16 : 4) : nullptr;
+  }
+
   for (int head = h_begin; head < h_end; ++head) {
     if (!PF) { ET_ATTN_LOAD_HEAD(head) }
     if (head != h_begin) __syncthreads();      // every wavefront is done with the previous head's tiles
@@ -491,8 +500,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
         }
       }
       // ---- write the lane's 16 features of its query's packed row --------------------------
-      const int tq = tok_of_pos[q];
-      if (tq >= 0) {
+      if (out_row[qi] != nullptr) {
         if constexpr (sizeof(T) == 2) {
           // o[j][r] is feature 16*g + 4*r + j: 16 consecutive features
           half8 v0, v1;
@@ -503,11 +511,11 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
               v0[4 * r + j] = f2h(o[j][r]);
               v1[4 * r + j] = f2h(o[j][2 + r]);
             }
-          T* orow = dst + (size_t)tq * H + head * kD + g * 16;
+          T* orow = out_row[qi] + head * kD;
           *reinterpret_cast<half8*>(orow) = v0;
           *reinterpret_cast<half8*>(orow + 8) = v1;
         } else {
-          T* orow = dst + (size_t)tq * H + head * kD + g * 4;
+          T* orow = out_row[qi] + head * kD;
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt) {
             typedef T out4 __attribute__((ext_vector_type(4)));
