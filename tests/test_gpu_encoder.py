@@ -377,6 +377,39 @@ def test_random_shapes_against_oracle(seed):
     _check(got, _oracle(w), mask, dtype)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_long_shapes_against_oracle(seed):
+    """One layer on randomly drawn shapes around the borders between the attention kernels (128, 256, 384, 512 keys)
+    and up to the 1024 keys the reference's softmax launch covers (cuda/attention.cu:345-356): holes in the mask, empty
+    sequences, attention masks unrelated to the input mask, both element types, against the oracle."""
+    rng = np.random.RandomState(2000 + seed)
+    dtype = ["fp16", "fp32"][seed % 2]
+    B = int(rng.randint(1, 5))
+    S = int(rng.choice([129, 255, 257, 300, 383, 384, 385, 511, 512, 513, 640, 777, 1000, 1024]))
+    heads = int(rng.choice([1, 2, 3]))
+    print("random long shape", seed, dtype, "B", B, "S", S, "heads", heads, flush=True)
+    wl = o.Workload("rndlong", 2000 + seed, dtype, 1, B, S, heads, 64, 4 * heads * 64, 1, S + 1)
+    if seed % 3 == 0:
+        mask = (rng.rand(B, S) < 0.7).astype(np.int32)
+        if B > 1:
+            mask[rng.randint(0, B)] = 0                       # an empty sequence
+        attr = (rng.rand(B, S, S) < 0.8).astype(np.float32)   # an attention mask unrelated to the input mask
+    else:
+        lens = rng.randint(1, S + 1, size=B)
+        lens[0] = S                                           # one sequence of full length
+        mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.int32)
+        attr = np.ascontiguousarray(np.broadcast_to(mask[:, None, :], (B, S, S))).astype(np.float32)
+    attr = o.rnd(attr, dtype)
+    x = o.rnd(rng.randn(B, S, wl.H), dtype)
+    weights = o.make_layer_weights(wl, rng, True)
+    w = dict(wl=wl, lens=None, mask=mask, attr_mask=attr, x=x, weights=weights)
+    got = run_encoder(w)
+    if mask.sum() == 0:
+        assert np.all(got == 0)
+        return
+    _check(got, _oracle(w), mask, dtype)
+
+
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 def test_cpp_host_gives_the_same_bits(tmp_path, dtype):
     """The C++ sample (csrc/encoder_example.cpp on include/et.hpp) against the Python mirror on the same problem."""
