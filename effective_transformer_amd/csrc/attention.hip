@@ -1594,6 +1594,7 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
 
   // ---- the additive bias of this half of the mask row: all loads of the row in flight before the first use -------
   float s[NKT][4];                                           // s[2 P], s[2 P + 1]: keys base + 8 g + 0..3, + 4..7 of pair P
+  // (1 - m) * -10000 as one fma: 1 - m is exact in float for a half m, so both forms round the same real number once
   {
     int g8 = g * 8;
     asm volatile("" : "+v"(g8));       // opaque: the clamped offsets are recomputed, not kept in registers
@@ -1608,11 +1609,11 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
         const int key0 = (kt_base + 2 * kp) * 16 + g8;
         if ((kt_base + 2 * kp + 2) * 16 <= seq_len) {        // wave-uniform: every key of the pair exists
 #pragma unroll
-          for (int j = 0; j < 8; ++j) s[2 * kp + (j >> 2)][j & 3] = (1.0f - (float)m8[kp][j]) * -10000.0f;
+          for (int j = 0; j < 8; ++j) s[2 * kp + (j >> 2)][j & 3] = __builtin_fmaf((float)m8[kp][j], 10000.0f, -10000.0f);
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j)
-            s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? (1.0f - (float)m8[kp][j]) * -10000.0f : -INFINITY;
+            s[2 * kp + (j >> 2)][j & 3] = key0 < seq_len ? __builtin_fmaf((float)m8[kp][j], 10000.0f, -10000.0f) : -INFINITY;
         }
       }
     } else {
@@ -1622,7 +1623,7 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const T m = mrow[min(key0 + j, seq_len - 1)];
-          s[2 * kp + (j >> 2)][j & 3] = key0 + j < seq_len ? (1.0f - (float)m) * -10000.0f : -INFINITY;
+          s[2 * kp + (j >> 2)][j & 3] = key0 + j < seq_len ? __builtin_fmaf((float)m, 10000.0f, -10000.0f) : -INFINITY;
         }
         if (kp % 4 == 3) __builtin_amdgcn_sched_barrier(0);
       }
