@@ -1,6 +1,6 @@
 """Benchmark of the padding-free BERT encoder on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--no-cpu] [--no-calibrate]
 
 A step is one pass Input -> L x Layer -> Output over one synthetic batch that is already
 resident in HBM.  Prints ONE JSON line: valid tokens/s (whole job), ms/step, the roofline of the
@@ -378,8 +378,10 @@ def main():
     ap.add_argument("--cpu-seqs", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--calibrate-mfma", action="store_true",
-                    help="also measure the MFMA rate the GPU sustains on zero and on random operands (fp16)")
+    ap.add_argument("--no-calibrate", action="store_true",
+                    help="skip the measurement of the MFMA rate the GPU sustains on zero and on random operands "
+                         "(fp16, about 0.3 s), which otherwise goes into `mfma_ceiling`")
+    ap.add_argument("--calibrate-mfma", action="store_true", help="kept for old command lines: the measurement is on by default")
     ap.add_argument("--calibrate-gemm", action="store_true",
                     help="also time the vendor library's GEMM (torch.matmul) on the four projection shapes")
     ap.add_argument("--fold-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
@@ -476,7 +478,7 @@ def main():
                     "measured": "HIP events around the kernel inside the layer's launch sequence, %d launches" % (4 * wl.layers),
                     "alone": alone, "traffic": measured_traffic(wl.name, dom)}
     ceiling = None
-    if a.calibrate_mfma:
+    if not a.no_calibrate and wl.dtype == "fp16":
         try:
             ceiling = mfma_ceiling()
             if roof is not None and roof["bound"] == "mfma" and wl.dtype == "fp16":

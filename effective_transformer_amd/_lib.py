@@ -31,7 +31,8 @@ class LayerWeights(C.Structure):
 class LayerPrepared(C.Structure):
     _fields_ = [("attr_kernel_Q_t", C.c_void_p), ("attr_kernel_K_t", C.c_void_p), ("attr_kernel_V_t", C.c_void_p),
                 ("attr_output_kernel_t", C.c_void_p), ("inter_kernel_t", C.c_void_p), ("output_kernel_t", C.c_void_p),
-                ("seq_start", C.c_void_p), ("warm", C.c_void_p), ("warm_bytes", C.c_size_t)]
+                ("seq_start", C.c_void_p), ("warm", C.c_void_p), ("warm_bytes", C.c_size_t),
+                ("seq_start_bytes", C.c_size_t)]
 
 
 class EmbeddingWeights(C.Structure):
@@ -64,7 +65,7 @@ SIGNATURES = {
                                 _vp, _sz, _vp, _ip]),
     "et_layer": (_i, [_vp, _i, C.POINTER(LayerWeights), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                       _vp, _sz, _vp]),
-    "et_sequence_starts": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "et_sequence_starts": (_i, [_vp, _vp, _vp, _i, _i, _vp, _sz, _vp]),
     "et_layer_with_prepared": (_i, [_vp, _i, C.POINTER(LayerWeights), C.POINTER(LayerPrepared), _vp, _vp, _vp, _vp, _vp,
                                     _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "et_first_token": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -80,7 +81,7 @@ SIGNATURES = {
     "et_transpose_rm_padding": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "et_attention": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _sz, _vp]),
     "et_attention_with_starts": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp,
-                                      _vp]),
+                                      _sz, _vp]),
     "et_gemm": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_gemm_bias_gelu": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "et_transpose_weight": (_i, [_vp, _i, _vp, _vp, _i, _i, _vp]),

@@ -1172,10 +1172,11 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, float scaler) {
+  static_assert(sizeof(T) == 4, "fp32 only: fp16 beyond 512 positions runs attention_wide_kernel");
   using Sm = LongSmem<T>;
   using C = Chunk16<T>;
   using V16 = typename C::vec;
-  constexpr int kQS = Sm::kQS, kVR = Sm::kVR, kVS = Sm::kVS;
+  constexpr int kQS = Sm::kQS, kVS = Sm::kVS;
   constexpr int kCpr = kD / C::kElems;
   constexpr int NKT = kSplitHalfTiles;
   constexpr int kChunks = NKT / kLongChunkTiles;             // 4 steps of 128 keys per half
@@ -1215,9 +1216,10 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
   auto src_off = [&](int t, int pos) -> size_t {
     return layout == 1 ? (size_t)t * packed_ld + head * kD : (((size_t)b * heads + head) * seq_len + pos) * kD;
   };
-  // rows [c0, c0 + 128) of `src`, zeros where no token sits: global memory -> registers, registers -> this half's
-  // buffer (row-major, stride `stride` elements).  The fp16 kernel fetches a chunk while the one before it is used.
-  auto fetch_rows = [&](const T* __restrict__ src, int c0, V16 (&r)[CPT]) {
+  // rows [c0, c0 + 128) of `src`, zeros where no token sits: global memory -> registers -> this half's buffer
+  // (row-major, stride `stride` elements)
+  auto stage_rows = [&](const T* __restrict__ src, T* lds, int stride, int c0) {
+    V16 r[CPT];
 #pragma unroll
     for (int k = 0; k < CPT; ++k) {
       const int i = tid_h + k * kAttnThreads;
@@ -1228,8 +1230,6 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
       for (int j = 0; j < C::kElems; ++j) r[k][j] = (T)0;
       if (tk >= 0) r[k] = *reinterpret_cast<const V16*>(src + src_off(tk, pos) + c * C::kElems);
     }
-  };
-  auto put_rows = [&](T* lds, int stride, const V16 (&r)[CPT]) {
 #pragma unroll
     for (int k = 0; k < CPT; ++k) {
       const int i = tid_h + k * kAttnThreads;
@@ -1237,14 +1237,6 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
       *reinterpret_cast<V16*>(lds + row * stride + c * C::kElems) = r[k];
     }
   };
-  auto stage_rows = [&](const T* __restrict__ src, T* lds, int stride, int c0) {
-    V16 r[CPT];
-    fetch_rows(src, c0, r);
-    put_rows(lds, stride, r);
-  };
-  constexpr bool kAhead = sizeof(T) == 2;                    // fp32: twice the registers per chunk, no room
-  auto half_has_tokens = [&](int ch) { return kt_base + ch * kLongChunkTiles < n_tiles; };
-  V16 pre[kAhead ? CPT : 1];
 
   const int qt = qblock * 4 + tile_w;                        // this wavefront's 16-query tile
   const bool active = qt < n_tiles;                          // wave-uniform
@@ -1254,27 +1246,13 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
   const bool vec_mask = (seq_len & 3) == 0;
 
   // Q operand of this lane (zeros for a query position without a token: its result is never stored)
-  half8 bqh[2];
   float bqf[16];
-  if constexpr (sizeof(T) == 2) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+  for (int i = 0; i < 4; ++i) {
+    float4v v4 = {0.f, 0.f, 0.f, 0.f};
+    if (tq >= 0) v4 = *reinterpret_cast<const float4v*>(q_src + src_off(tq, q) + g * 16 + i * 4);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) bqh[ks][j] = (_Float16)0;
-      if (tq >= 0) bqh[ks] = *reinterpret_cast<const half8*>(q_src + src_off(tq, q) + ks * 32 + g * 8);
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float4v v4 = {0.f, 0.f, 0.f, 0.f};
-      if (tq >= 0) v4 = *reinterpret_cast<const float4v*>(q_src + src_off(tq, q) + g * 16 + i * 4);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) bqf[i * 4 + j] = v4[j];
-    }
-  }
-
-  if constexpr (kAhead) {
-    if (half_has_tokens(0)) fetch_rows(k_src, kt_base * 16, pre);
+    for (int j = 0; j < 4; ++j) bqf[i * 4 + j] = v4[j];
   }
 
   // ---- the additive bias of this half of the mask row (no branch between the loads) -------------------------
@@ -1306,45 +1284,22 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
     if (ch * kLongChunkTiles >= n_tiles) break;                          // workgroup-uniform: no token in either half
     const bool chunk_has_tokens = kt_base + ch * kLongChunkTiles < n_tiles;   // uniform over this half's 4 wavefronts
     __syncthreads();                                                     // previous chunks fully consumed
-    if (chunk_has_tokens) {
-      if constexpr (kAhead) {
-        put_rows(Ks, kQS, pre);
-      } else {
-        stage_rows(k_src, Ks, kQS, (kt_base + ch * kLongChunkTiles) * 16);
-      }
-    }
+    if (chunk_has_tokens) stage_rows(k_src, Ks, kQS, (kt_base + ch * kLongChunkTiles) * 16);
     __syncthreads();
-    if constexpr (kAhead) {
-      if (ch + 1 < kChunks && half_has_tokens(ch + 1))
-        fetch_rows(k_src, (kt_base + (ch + 1) * kLongChunkTiles) * 16, pre);
-      else if (half_has_tokens(0) && (ch + 1 == kChunks || (ch + 1) * kLongChunkTiles >= n_tiles))
-        fetch_rows(v_src, kt_base * 16, pre);                            // last K chunk of the workgroup: V comes next
-    }
     if (active && chunk_has_tokens) {
 #pragma unroll
       for (int kc = 0; kc < kLongChunkTiles; ++kc) {
         const int ktl = ch * kLongChunkTiles + kc;
         if (kt_base + ktl < n_tiles) {
           float4v acc = {0.f, 0.f, 0.f, 0.f};
-          if constexpr (sizeof(T) == 2) {
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-              const half8 a = *reinterpret_cast<const half8*>(Ks + (kc * 16 + l16) * kQS + ks * 32 + g * 8);
-              acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bqh[ks], acc, 0, 0, 0);
-            }
-          } else {
+          for (int i = 0; i < 4; ++i) {
+            const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kc * 16 + l16) * kQS + g * 16 + i * 4);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float4v a4 = *reinterpret_cast<const float4v*>(Ks + (kc * 16 + l16) * kQS + g * 16 + i * 4);
-#pragma unroll
-              for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bqf[i * 4 + j], acc, 0, 0, 0);
-            }
+            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], bqf[i * 4 + j], acc, 0, 0, 0);
           }
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float sc = sizeof(T) == 2 ? h2f(f2h(acc[r])) : acc[r];   // the score is stored in the element type
-            s[ktl][r] = sc * scaler + s[ktl][r];
-          }
+          for (int r = 0; r < 4; ++r) s[ktl][r] = acc[r] * scaler + s[ktl][r];
         }
       }
     }
@@ -1397,71 +1352,30 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
     const bool chunk_has_tokens = kt_base + ch * kLongChunkTiles < n_tiles;
     __syncthreads();
     if (chunk_has_tokens) {
-      if constexpr (kAhead) {
-        put_rows(Vs, kVR, pre);
-      } else {
-        // fp32 keeps V^T: feature rows, key columns
+      // V^T in LDS: feature rows, key columns
 #pragma unroll
-        for (int k = 0; k < CPT; ++k) {
-          const int i = tid_h + k * kAttnThreads;
-          const int row = i / kCpr, c = i - row * kCpr;
-          const int pos = (kt_base + ch * kLongChunkTiles) * 16 + row;
-          const int tk = pos < kSplitKeys ? tok_of_pos[pos] : -1;
-          V16 r = {0.f, 0.f, 0.f, 0.f};
-          if (tk >= 0) r = *reinterpret_cast<const V16*>(v_src + src_off(tk, pos) + c * C::kElems);
+      for (int k = 0; k < CPT; ++k) {
+        const int i = tid_h + k * kAttnThreads;
+        const int row = i / kCpr, c = i - row * kCpr;
+        const int pos = (kt_base + ch * kLongChunkTiles) * 16 + row;
+        const int tk = pos < kSplitKeys ? tok_of_pos[pos] : -1;
+        V16 r = {0.f, 0.f, 0.f, 0.f};
+        if (tk >= 0) r = *reinterpret_cast<const V16*>(v_src + src_off(tk, pos) + c * C::kElems);
 #pragma unroll
-          for (int j = 0; j < C::kElems; ++j) Vs[(c * C::kElems + j) * kVS + row] = r[j];
-        }
+        for (int j = 0; j < C::kElems; ++j) Vs[(c * C::kElems + j) * kVS + row] = r[j];
       }
     }
     __syncthreads();
-    if constexpr (kAhead) {
-      if (ch + 1 < kChunks && half_has_tokens(ch + 1)) fetch_rows(v_src, (kt_base + (ch + 1) * kLongChunkTiles) * 16, pre);
-    }
     if (!active || !chunk_has_tokens) continue;
-    if constexpr (sizeof(T) == 2) {
 #pragma unroll
-      for (int kp = 0; kp < kLongChunkTiles / 2; ++kp) {
-        const int ktl = ch * kLongChunkTiles + 2 * kp;
-        if (kt_base + ktl < n_tiles) {
-          half8 p;
+    for (int kc = 0; kc < kLongChunkTiles; ++kc) {
+      const int ktl = ch * kLongChunkTiles + kc;
+      if (kt_base + ktl < n_tiles) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            p[r] = f2h(s[ktl][r]);
-            p[4 + r] = f2h(s[ktl + 1][r]);
-          }
-          typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-          typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-          u2 raw[8];
+        for (int dt = 0; dt < 4; ++dt) {
+          const float4v a4 = *reinterpret_cast<const float4v*>(Vs + (dt * 16 + l16) * kVS + kc * 16 + g * 4);
 #pragma unroll
-          for (int kk = 0; kk < 8; ++kk) {
-            const int key = kp * 32 + (kk >> 2) * 16 + g * 4 + (kk & 3);
-            raw[kk] = *reinterpret_cast<const u2*>(Vs + key * kVR + l16 * 4);
-          }
-#pragma unroll
-          for (int jj = 0; jj < 2; ++jj) {
-            u4 lo, hi;
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-              lo[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x05040100u);
-              hi[q4] = __builtin_amdgcn_perm(raw[2 * q4 + 1][jj], raw[2 * q4][jj], 0x07060302u);
-            }
-            o[2 * jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, lo), p, o[2 * jj], 0, 0, 0);
-            o[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, hi), p, o[2 * jj + 1], 0, 0, 0);
-          }
-        }
-      }
-    } else {
-#pragma unroll
-      for (int kc = 0; kc < kLongChunkTiles; ++kc) {
-        const int ktl = ch * kLongChunkTiles + kc;
-        if (kt_base + ktl < n_tiles) {
-#pragma unroll
-          for (int dt = 0; dt < 4; ++dt) {
-            const float4v a4 = *reinterpret_cast<const float4v*>(Vs + (dt * 16 + l16) * kVS + kc * 16 + g * 4);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[ktl][r], o[dt], 0, 0, 0);
-          }
+          for (int r = 0; r < 4; ++r) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], s[ktl][r], o[dt], 0, 0, 0);
         }
       }
     }
@@ -1482,27 +1396,13 @@ __global__ __launch_bounds__(kSplitThreads) void attention_split_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) o[dt][r] += other[r];
     }
-    if constexpr (sizeof(T) == 2) {
-      half8 v0, v1;
+    T* orow = dst + (size_t)tq * H + head * kD + g * 4;
 #pragma unroll
-      for (int r = 0; r < 2; ++r)
+    for (int dt = 0; dt < 4; ++dt) {
+      float4v v;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v0[4 * r + j] = f2h(o[j][r]);
-          v1[4 * r + j] = f2h(o[j][2 + r]);
-        }
-      T* orow = dst + (size_t)tq * H + head * kD + g * 16;
-      *reinterpret_cast<half8*>(orow) = v0;
-      *reinterpret_cast<half8*>(orow + 8) = v1;
-    } else {
-      T* orow = dst + (size_t)tq * H + head * kD + g * 4;
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        float4v v;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = o[dt][r];
-        *reinterpret_cast<float4v*>(orow + dt * 16) = v;
-      }
+      for (int r = 0; r < 4; ++r) v[r] = o[dt][r];
+      *reinterpret_cast<float4v*>(orow + dt * 16) = v;
     }
   }
 }
@@ -1785,24 +1685,25 @@ __global__ __launch_bounds__(kSplitThreads) void attention_wide_kernel(
 #endif
 }
 
+// 512 < seq_len <= 1024, head size 64: fp32 runs the chunked split kernel, fp16 the kernel with the whole sequence in LDS
 template <typename T>
 void attention_split_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                             void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                             float scaler, hipStream_t stream) {
-  const size_t smem = 2 * LongSmem<T>::kTileBytes + (size_t)kSplitKeys * sizeof(int) + 2 * 4 * 2 * 16 * sizeof(float);
   dim3 grid((seq_len + 63) / 64, heads, batch);              // blocks of 64 queries that can hold a token
   if constexpr (sizeof(T) == 2) {
     allow_dynamic_lds(reinterpret_cast<const void*>(attention_wide_kernel), kWideSmem);
     attention_wide_kernel<<<grid, kSplitThreads, kWideSmem, stream>>>(
         (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, layout, packed_ld, (const _Float16*)attr_mask,
         (_Float16*)dst, seq_start, word_idx, batch, seq_len, heads, scaler);
-    return;
+  } else {
+    const size_t smem = 2 * LongSmem<T>::kTileBytes + (size_t)kSplitKeys * sizeof(int) + 2 * 4 * 2 * 16 * sizeof(float);
+    auto kern = attention_split_kernel<T>;
+    allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem);
+    kern<<<grid, kSplitThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
+                                                (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch, seq_len, heads,
+                                                scaler);
   }
-  auto kern = attention_split_kernel<T>;
-  allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem);
-  kern<<<grid, kSplitThreads, smem, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
-                                              (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch, seq_len, heads,
-                                              scaler);
 }
 
 // ------------------------------------------------------------------------------------------

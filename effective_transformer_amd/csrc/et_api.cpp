@@ -49,24 +49,30 @@ hipError_t take_attribute_error() {
 
 namespace {
 
-// Scratch of et_input_static: the tile totals of the mask scan (one int32 per tile of 1024 positions) for up to
-// kStaticMaxPositions positions.  Every GPU the library runs on holds its own copy of the array until the process
-// ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use is looked
-// up once per device (et_create) and kept in static_scratch_ptr.
 // The persistent GEMM stores C with plain stores while the matrices of a layer (resp. A and C of a stand-alone call)
 // are small enough to be found in the 256 MB last-level cache by the kernels that read them next, and with non-temporal
 // stores beyond.  12-layer BERT-base, fp16: plain stores -6 % at 4000 tokens, -2.4 % at 15900, +-0.5 % at 20000,
 // +2 % at 30000 and 40000; 24-layer BERT-large at 13100 tokens: -0.4 %.
 constexpr double kCachedLayerBytes = 320.0 * 1048576.0;
 constexpr double kCachedCallBytes = 96.0 * 1048576.0;
+// While the layer's matrices stay below this, weights requested ahead of FFN-up survive until FFN-down reads them.
 constexpr double kWarmLayerBytes = 256.0 * 1048576.0;
-constexpr int kStaticScratchWords = 1024;
+
+// Scratch of et_input_static: the tile totals of the mask scan (one int32 per tile of 1024 positions) for up to
+// kStaticMaxPositions positions, in kStaticSlots independent slots.  A handle takes a free slot of its device when it
+// is created and gives it back when it is destroyed, so that two handles never share tile totals; the handles beyond
+// kStaticSlots per device have none.  Every GPU the library runs on holds its own copy of the array until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use
+// is looked up once per device (et_create) and kept in static_scratch_ptr.
+constexpr int kStaticSlotWords = 1024;
+constexpr int kStaticSlots = 8;
 constexpr int kStaticMaxPositions = 1024 * 1024;
-static __device__ __align__(256) int32_t scratch[kStaticScratchWords];
+static __device__ __align__(256) int32_t scratch[kStaticSlots * kStaticSlotWords];
 
 constexpr int kMaxDevices = 64;
 std::mutex static_scratch_mu;
 int32_t* static_scratch_ptr[kMaxDevices] = {};
+unsigned static_slots_taken[kMaxDevices] = {};       // bit s: slot s of the device belongs to a live handle
 
 // Looks up this device's copy of `scratch` (the device must be current).  Called by et_create.
 hipError_t resolve_static_scratch(int device) {
@@ -80,26 +86,54 @@ hipError_t resolve_static_scratch(int device) {
   return hipSuccess;
 }
 
+// A free slot of the device for a new handle, -1 when all are taken.
+int take_static_slot(int device) {
+  std::lock_guard<std::mutex> lock(static_scratch_mu);
+  for (int s = 0; s < kStaticSlots; ++s)
+    if (!(static_slots_taken[device] & (1u << s))) {
+      static_slots_taken[device] |= 1u << s;
+      return s;
+    }
+  return -1;
+}
+
+void release_static_slot(int device, int slot) {
+  if (slot < 0 || device < 0 || device >= kMaxDevices) return;
+  std::lock_guard<std::mutex> lock(static_scratch_mu);
+  static_slots_taken[device] &= ~(1u << slot);
+}
+
 }  // namespace
 
 struct et_context {
   int device = 0;
-  std::mutex mu;
-  std::string last_error;
+  std::mutex mu;                   // serialises the calls on this handle
+  std::mutex err_mu;               // guards last_error alone: a failure may be recorded before `mu` is taken
+  std::string last_error;          // the last failure on this handle by any thread
+  // et_input_static: the handle's slot of the device's static scratch (-1: none), and the stream its calls are bound to
+  int static_slot = -1;
+  bool static_stream_set = false;
+  hipStream_t static_stream = nullptr;
 };
 
 namespace {
 
+// The calling thread's last failure and the handle it happened on (null: without a handle).  et_last_error prefers it,
+// so a thread reads its own message whatever other threads do on the same handle in the meantime.
 thread_local std::string tls_error;
+thread_local et_handle tls_error_handle = nullptr;
+thread_local std::string tls_error_copy;      // et_last_error's copy of another thread's message
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 et_status fail(et_handle h, et_status s, const std::string& msg) {
   std::string full = std::string("[ET][ERROR] ") + et_status_string(s) + ": " + msg;
-  if (h)
+  if (h) {
+    std::lock_guard<std::mutex> lock(h->err_mu);
     h->last_error = full;
-  else
-    tls_error = full;
+  }
+  tls_error = std::move(full);
+  tls_error_handle = h;
   return s;
 }
 
@@ -234,17 +268,26 @@ et_status et_create(et_handle* out, int device) {
   et_context* c = new (std::nothrow) et_context();
   if (!c) return fail(nullptr, ET_RUNTIME_ERROR, "out of host memory");
   c->device = device;
+  c->static_slot = device < kMaxDevices ? take_static_slot(device) : -1;
   *out = c;
   return ET_OK;
 }
 
 et_status et_destroy(et_handle h) {
   if (!h) return ET_OK;
+  release_static_slot(h->device, h->static_slot);
+  if (tls_error_handle == h) tls_error_handle = nullptr;
   delete h;
   return ET_OK;
 }
 
-const char* et_last_error(et_handle h) { return h ? h->last_error.c_str() : tls_error.c_str(); }
+const char* et_last_error(et_handle h) {
+  if (tls_error_handle == h) return tls_error.c_str();       // this thread's own last failure (on h, or without a handle)
+  if (!h) return "";
+  std::lock_guard<std::mutex> lock(h->err_mu);
+  tls_error_copy = h->last_error;
+  return tls_error_copy.c_str();
+}
 
 size_t et_input_workspace_bytes(int batch_size, int seq_len) {
   if (batch_size < 1 || seq_len < 1) return 0;
@@ -302,17 +345,35 @@ et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, 
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && mask && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
   if ((long)batch_size * seq_len > kStaticMaxPositions ||
-      et::scan_scratch_words(batch_size * seq_len) > (size_t)kStaticScratchWords)
+      et::scan_scratch_words(batch_size * seq_len) > (size_t)kStaticSlotWords)
     return fail(h, ET_UNSUPPORTED,
                 "et_input_static holds scratch for batch_size * seq_len <= 1048576 positions; larger batches go "
                 "through et_input with a caller workspace");
+  if (h->static_slot < 0)
+    return fail(h, ET_UNSUPPORTED,
+                "this handle holds no slot of the static scratch (at most 8 live handles per GPU do); use et_input");
   const size_t row_bytes = (size_t)head_num * size_per_head * et::elem_size(to_dt(dtype));
   if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
   if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
     return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
   int32_t* scratch_dev = h->device < kMaxDevices ? static_scratch_ptr[h->device] : nullptr;
   if (!scratch_dev) return fail(h, ET_RUNTIME_ERROR, "no static scratch on this device");
+  scratch_dev += (size_t)h->static_slot * kStaticSlotWords;
+  // Calls that share a slot must not overlap on the GPU.  Calls queued on one stream cannot; a call on another stream
+  // is accepted only once everything queued on the previous one has finished.
   hipStream_t st = (hipStream_t)stream;
+  if (h->static_stream_set && h->static_stream != st) {
+    // (any other answer than "not ready", e.g. for a stream that no longer exists, lets the call through)
+    const hipError_t q = hipStreamQuery(h->static_stream);
+    if (q != hipSuccess) (void)hipGetLastError();
+    if (q == hipErrorNotReady) {
+      return fail(h, ET_INVALID_ARGUMENT,
+                  "et_input_static: the stream of this handle's previous call still has work in flight, and calls on "
+                  "two streams would share the handle's scratch slot; wait for that stream or use a second handle");
+    }
+  }
+  h->static_stream_set = true;
+  h->static_stream = st;
   // the scan writes every tile total it later reads, so nothing of the previous call's contents has to be cleared
   et::launch_scan_index(mask, batch_size * seq_len, nullptr, batch_idx, word_idx, valid_word_num_dev, seq_len,
                         scratch_dev, st);
@@ -374,12 +435,14 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* w, const
 }
 
 et_status et_sequence_starts(et_handle h, const int32_t* batch_idx, const int32_t* valid_word_num_dev, int batch_size,
-                             int seq_len, int32_t* seq_start, void* stream) {
+                             int seq_len, int32_t* seq_start, size_t seq_start_bytes, void* stream) {
   Entry entry(h);
   et_status s = entry.status;
   if (s != ET_OK) return s;
   if ((s = dims_ok(h, batch_size, seq_len, 1, 1)) != ET_OK) return s;
   ET_REQUIRE(h, batch_idx && valid_word_num_dev && seq_start, "null tensor pointer");
+  if (seq_start_bytes < et_seq_workspace_bytes(batch_size))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "the sequence table needs et_seq_workspace_bytes(batch_size)");
   et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, seq_start, (hipStream_t)stream);
   return check_launch(h, "sequence starts");
 }
@@ -435,8 +498,10 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   // The large-M fp16 GEMM reads k-contiguous weights with fewer LDS instructions.  Where the caller prepared such
   // copies they are used wherever that kernel runs; otherwise the wide projections get a transposed copy in the
   // workspace on every call (the caller's weights stay as they are).
-  static const et_layer_prepared kNoPrep = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+  static const et_layer_prepared kNoPrep = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
   const et_layer_prepared& pp = prep ? *prep : kNoPrep;
+  if (pp.seq_start && pp.seq_start_bytes < et_seq_workspace_bytes(B))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "et_layer_prepared.seq_start needs et_seq_workspace_bytes(batch_size) bytes");
   ET_REQUIRE(h, (pp.attr_kernel_Q_t != nullptr) == (pp.attr_kernel_K_t != nullptr) &&
                     (pp.attr_kernel_Q_t != nullptr) == (pp.attr_kernel_V_t != nullptr),
              "prepared Q, K and V kernels go together");
@@ -710,14 +775,15 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
   }
   return et_attention_with_starts(h, dtype, q, k, v, qkv_layout, packed_ld, attr_mask, dst, valid_word_num_dev,
                                   batch_size, seq_len, head_num, size_per_head, batch_idx, word_idx, nullptr,
-                                  (int32_t*)workspace, stream);
+                                  (int32_t*)workspace, workspace_bytes, stream);
 }
 
 et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v,
                                    int qkv_layout, int packed_ld, const void* attr_mask, void* dst,
                                    const int32_t* valid_word_num_dev, int batch_size, int seq_len, int head_num,
                                    int size_per_head, const int32_t* batch_idx, const int32_t* word_idx,
-                                   const int32_t* seq_start, int32_t* seq_start_scratch, void* stream) {
+                                   const int32_t* seq_start, int32_t* seq_start_scratch, size_t seq_table_bytes,
+                                   void* stream) {
   Entry entry(h);
   et_status s = entry.status;
   if (s != ET_OK) return s;
@@ -727,6 +793,8 @@ et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, c
   ET_REQUIRE(h, qkv_layout == 0 || qkv_layout == 1, "qkv_layout must be 0 (padded) or 1 (packed)");
   ET_REQUIRE(h, qkv_layout == 0 || packed_ld >= head_num * size_per_head, "packed_ld smaller than the hidden size");
   ET_REQUIRE(h, seq_start != nullptr || seq_start_scratch != nullptr, "null sequence start table");
+  if (seq_table_bytes < et_seq_workspace_bytes(batch_size))
+    return fail(h, ET_WORKSPACE_TOO_SMALL, "the sequence table needs et_seq_workspace_bytes(batch_size)");
   if ((s = batch_fits_grid(h, batch_size)) != ET_OK) return s;
   if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
     return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 in multiples of 16 bytes and seq_len <= 1024");

@@ -171,8 +171,9 @@ __global__ __launch_bounds__(kLnThreads) void bias_residual_layernorm_kernel(
       }
     }
   }
-  // never true (rows >= 0); keeps the requests above alive
-  if (rows < 0 && (warm0 ^ warm1) == 0x9e3779b9u) out[0] = (T)0;
+  // The requested words are consumed here, behind the row loop, by an empty instruction sequence: the loads cannot be
+  // dropped, and nothing that depends on a corrupt row count decides whether they stay.
+  asm volatile("" ::"v"(warm0), "v"(warm1));
 }
 
 // ------------------------------------------------------------------------------------------

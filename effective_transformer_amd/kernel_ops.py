@@ -96,7 +96,7 @@ def attention(q, k, v, layout: int, packed_ld: int, attr_mask, valid_word_num, B
     if seq_start is not None:
         _call("et_attention_with_starts", dev, _dtype_code(attr_mask.dtype), _p(q), _p(k), _p(v), layout, packed_ld,
               _p(attr_mask), _p(dst), _p(valid_word_num), B, S, heads, d, _p(batch_idx), _p(word_idx), _p(seq_start), None,
-              _stream())
+              seq_start.numel() * seq_start.element_size(), _stream())
         return dst
     ws = _workspace(dev, "seq", lib.et_seq_workspace_bytes(B))
     _call("et_attention", dev, _dtype_code(attr_mask.dtype), _p(q), _p(k), _p(v), layout, packed_ld, _p(attr_mask),

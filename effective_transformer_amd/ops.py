@@ -44,12 +44,13 @@ _scope = threading.local()      # .owner: set while a GraphedEncoder warms up an
 
 
 def _workspace(device: torch.device, kind: str, nbytes: int) -> torch.Tensor:
-    """One scratch buffer per (GPU, stream, kind, owner), grown on demand: calls queued on one stream run in order and
-    may share it, calls on different streams get their own, and so does every captured graph (a graph keeps the
-    addresses it was captured with, and replays of two graphs on different streams may overlap).  Within one such key
-    the contract is one stream of calls: the layer op keeps its intermediate tensors there between its launches."""
+    """One scratch buffer per (GPU, stream, kind, owner, host thread), grown on demand: calls queued on one stream by
+    one thread run in order and may share it; calls on different streams get their own, so does every captured graph
+    (a graph keeps the addresses it was captured with, and replays of two graphs on different streams may overlap),
+    and so does every host thread (the layer op keeps its intermediate tensors there between the calls of one encoder
+    pass, and two threads' passes interleave on a shared stream call by call)."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    key = (idx, torch.cuda.current_stream(idx).cuda_stream, kind, getattr(_scope, "owner", None))
+    key = (idx, torch.cuda.current_stream(idx).cuda_stream, kind, getattr(_scope, "owner", None), threading.get_ident())
     with _lock:
         ws = _workspaces.get(key)
         if ws is None or ws.numel() < nbytes:
@@ -283,6 +284,7 @@ def effective_transformer(from_tensor: torch.Tensor, to_tensor: torch.Tensor, at
         if weights.prepared is not None:
             C.pointer(prep)[0] = weights.prepared
         prep.seq_start = seq_start.data_ptr() if seq_start is not None else None
+        prep.seq_start_bytes = seq_start.numel() * seq_start.element_size() if seq_start is not None else 0
         st = lib.et_layer_with_prepared(h, code, C.byref(weights.struct), C.byref(prep), _p(from_tensor), _p(to_tensor),
                                         _p(attr_mask), _p(valid_word_num), _p(batch_idx), _p(word_idx), _p(out), B,
                                         from_seq_len, to_seq_len, head_num, size_per_head, valid_word_num_hint, _p(ws),
@@ -301,10 +303,11 @@ def sequence_starts(valid_word_num: torch.Tensor, batch_idx: torch.Tensor, batch
     words = lib.et_seq_workspace_bytes(batch_size) // 4
     if out is None:
         out = torch.empty(words, dtype=torch.int32, device=batch_idx.device)
-    elif out.numel() < 2 * batch_size + 1:
-        raise ValueError("the sequence table holds 2 * batch_size + 1 int32")
+    elif out.dtype != torch.int32:
+        raise TypeError("the sequence table is int32")
     h = handle(batch_idx.device)
-    _lib.check(lib.et_sequence_starts(h, _p(batch_idx), _p(valid_word_num), batch_size, seq_len, _p(out), _stream()), h)
+    _lib.check(lib.et_sequence_starts(h, _p(batch_idx), _p(valid_word_num), batch_size, seq_len, _p(out),
+                                      out.numel() * 4, _stream()), h)
     return out
 
 
@@ -369,7 +372,10 @@ class EffectiveTransformerEncoder:
                     w.prepared.warm = nxt.warm_block.data_ptr()
                     w.prepared.warm_bytes = nxt.warm_block.numel() * 2
                     self._warm_refs.append(nxt.warm_block)
-        self._bufs: Dict[Tuple[int, ...], Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+        # ping-pong activations, sequence table and the pinned count, per (activation shape, stream, host thread): two
+        # threads or streams that run this encoder at the same time each have their own
+        self._bufs: Dict[tuple, list] = {}
+        self._bufs_lock = threading.Lock()
 
     @classmethod
     def from_checkpoint(cls, path: str, head_num: int, size_per_head: int, dtype: torch.dtype, device="cuda",
@@ -404,19 +410,24 @@ class EffectiveTransformerEncoder:
         behind the launches of the first layer, which is sized for B*S rows and bounded on the device: the GPU never
         idles for the read-back (waiting right after the input op left it without work for 0.13-0.19 ms per batch)."""
         hn, d = self.head_num, self.size_per_head
-        key = tuple(x.shape)
-        bufs = self._bufs.get(key)
+        key = (tuple(x.shape), torch.cuda.current_stream(x.device).cuda_stream, threading.get_ident(),
+               getattr(_scope, "owner", None))
+        with self._bufs_lock:
+            bufs = self._bufs.get(key)
         if bufs is None:
-            bufs = (torch.empty_like(x), torch.empty_like(x),
-                    torch.empty(2 * B + 1, dtype=torch.int32, device=x.device),
-                    torch.empty(1, dtype=torch.int32, pin_memory=True))
-            self._bufs[key] = bufs
+            # (the pinned word for the count is made on first use: a pass under graph capture never reads the count back)
+            bufs = [torch.empty_like(x), torch.empty_like(x),
+                    torch.empty(_lib.load().et_seq_workspace_bytes(B) // 4, dtype=torch.int32, device=x.device), None]
+            with self._bufs_lock:
+                self._bufs[key] = bufs
         T, copied = -1, None
         if not sync_count and rows_bound is not None:
             if not 0 < rows_bound <= B * S:
                 raise ValueError("rows_bound must be in 1 .. batch * seq_len")
             T = int(rows_bound)
         if sync_count and len(self.layers) > 1:
+            if bufs[3] is None:
+                bufs[3] = torch.empty(1, dtype=torch.int32, pin_memory=True)
             bufs[3].copy_(vwn, non_blocking=True)
             copied = torch.cuda.Event()
             copied.record()
@@ -456,30 +467,38 @@ class GraphedEncoder:
         self.x = from_tensor.clone()
         self.mask = input_mask.clone()
         self.attn = attention_mask.clone()
-        # warm-up outside the capture: workspaces, kernel attributes and the output buffers get created here.  The
-        # workspaces and the encoder's ping-pong buffers made under this owner belong to this graph alone.
+        # warm-up outside the capture (kernel attributes, allocator pools), on a side stream; its buffers are dropped
+        # again.  The workspaces and the encoder's ping-pong buffers made under this owner during the capture come from
+        # the graph's own memory pool, belong to this graph alone and are kept alive with it.
         _scope.owner = id(self)
-        saved_bufs, enc._bufs = enc._bufs, {}
+
+        def drop_owned():
+            with enc._bufs_lock:
+                for key in [k for k in enc._bufs if k[3] == id(self)]:
+                    del enc._bufs[key]
+            with _lock:
+                for key in [k for k in _workspaces if k[3] == id(self)]:
+                    del _workspaces[key]
+
         try:
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 for _ in range(2):
                     enc(self.x, self.mask, self.attn, sync_count=False, rows_bound=max_valid_tokens)
-                self._held = [ws for key, ws in list(_workspaces.items()) if key[3] == id(self)]
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
+            drop_owned()
             self.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self.graph):
                 self.out = enc(self.x, self.mask, self.attn, sync_count=False, rows_bound=max_valid_tokens)
-            self._held += [ws for key, ws in list(_workspaces.items()) if key[3] == id(self)]
-            self._held += [t for bufs in enc._bufs.values() for t in bufs]
+            with _lock:
+                self._held = [ws for key, ws in _workspaces.items() if key[3] == id(self)]
+            with enc._bufs_lock:
+                self._held += [t for key, bufs in enc._bufs.items() if key[3] == id(self) for t in bufs if t is not None]
         finally:
             _scope.owner = None
-            enc._bufs = saved_bufs
-            with _lock:
-                for key in [k for k in _workspaces if k[3] == id(self)]:
-                    del _workspaces[key]
+            drop_owned()
 
     def __call__(self, from_tensor=None, input_mask=None, attention_mask=None, check_mask: bool = True) -> torch.Tensor:
         """Copies the given tensors into the graph's inputs (None = keep the previous ones), replays, and returns the

@@ -49,8 +49,10 @@ typedef struct et_context* et_handle;
 et_status et_create(et_handle* out, int device);
 et_status et_destroy(et_handle h);
 /* Message of the last failing call on `h` (or, when h is NULL, of the last call on this thread that failed without a
- * handle: et_create, a NULL handle argument).  Never NULL.  The handle's message is rewritten by the next failing call
- * on it: with several threads on one handle, read it before another thread's call can fail. */
+ * handle: et_create, a NULL handle argument).  Never NULL.  With several threads on one handle every thread reads the
+ * message of ITS OWN last failing call as long as that call was its most recent failure; a thread that has not failed
+ * on `h` gets the handle's last message from any thread.  The pointer stays valid until the calling thread's next
+ * failing call or next et_last_error. */
 const char* et_last_error(et_handle h);
 const char* et_status_string(et_status s);
 /* 1 when the library was built for the architecture of `device` and a kernel runs there. */
@@ -101,11 +103,15 @@ et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const i
 
 /* et_input for callers that cannot allocate device memory or hand over a workspace (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels, same
- * outputs as et_input bit for bit; the scan's scratch (one int32 per 1024 mask positions) lives in a 4 KB array
- * inside the library's device image, one copy per GPU for the life of the process, so the call takes no workspace and
+ * outputs as et_input bit for bit; the scan's scratch (one int32 per 1024 mask positions) lives in an array
+ * inside the library's device image (32 KB), one copy per GPU for the life of the process, so the call takes no workspace and
  * allocates nothing.  Limit: batch_size * seq_len <= 1048576 positions (ET_UNSUPPORTED beyond; use et_input).  Never
- * synchronises (no host count).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
- * (different streams or handles) race; calls ordered on one stream are safe. */
+ * synchronises (no host count).  The array is cut into 8 slots; a handle takes a free slot of its GPU in et_create and
+ * returns it in et_destroy (a ninth live handle on one GPU has none: ET_UNSUPPORTED), so calls on different handles
+ * never share scratch.  The calls of ONE handle do: queued on one stream they run in order; a call on another stream
+ * than the handle's previous one is refused with ET_INVALID_ARGUMENT while that previous stream still has work in
+ * flight.  Replays of captured graphs that hold such calls are not seen by that check: replays of one handle's calls
+ * that overlap on the GPU race. */
 et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, const int32_t* mask,
                           void* to_tensor, int32_t* valid_word_num_dev, int32_t* batch_idx, int32_t* word_idx,
                           int batch_size, int seq_len, int head_num, int size_per_head, void* stream);
@@ -134,8 +140,9 @@ et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
  *   *_t: the dense kernel handed over [out,in] (k-contiguous), i.e. et_transpose_weight of the [in,out] tensor, fp16
  *        only.  Used where et_layer would run its large-M GEMM (it then skips its per-call transposition; Q, K and V
  *        go together); ignored for batches that run the small-M kernels, which read the [in,out] tensors.
- *   seq_start: the sequence table et_sequence_starts wrote for THIS batch (et_seq_workspace_bytes(batch_size) bytes);
- *        the same table serves every layer of the batch.
+ *   seq_start, seq_start_bytes: the sequence table et_sequence_starts wrote for THIS batch and the size of its buffer
+ *        (at least et_seq_workspace_bytes(batch_size), ET_WORKSPACE_TOO_SMALL below); the same table serves every
+ *        layer of the batch.
  *   warm, warm_bytes: a region that the layer's last kernel requests line by line on its way, so that whoever reads it
  *        next finds it in the last-level cache: the k-contiguous copies of the NEXT layer's attention kernels, whose
  *        GEMMs would otherwise wait for weights last read a whole batch ago.  Only used for batches large enough that
@@ -150,15 +157,17 @@ typedef struct et_layer_prepared {
   const int32_t* seq_start;          /* [2B+1] */
   const void* warm;                  /* see above; 128-byte aligned */
   size_t warm_bytes;
+  size_t seq_start_bytes;            /* bytes behind seq_start (checked when seq_start is set) */
 } et_layer_prepared;
 
 /* The sequence table of a batch, from the index arrays et_input produced: seq_start[b] = first packed row of sequence
  * b for b in [0,B), seq_start[B] = T, followed by the B sequence numbers in the order the attention kernels serve them
  * (by length, longest first: workgroups of similar duration run side by side and the long ones start first).
- * seq_start must hold et_seq_workspace_bytes(batch_size) bytes (2 B + 1 int32).  No counterpart in the reference (its
- * attention works on padded buffers). */
+ * seq_start must hold et_seq_workspace_bytes(batch_size) bytes (2 B + 1 int32); seq_start_bytes is the size of the
+ * caller's buffer, ET_WORKSPACE_TOO_SMALL when it is less.  No counterpart in the reference (its attention works on
+ * padded buffers). */
 et_status et_sequence_starts(et_handle h, const int32_t* batch_idx, const int32_t* valid_word_num_dev, int batch_size,
-                             int seq_len, int32_t* seq_start, void* stream);
+                             int seq_len, int32_t* seq_start, size_t seq_start_bytes, void* stream);
 
 /* et_layer with prepared data (see et_layer_prepared; NULL = et_layer).  Same results, bit for bit. */
 et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_weights* weights,
@@ -284,14 +293,15 @@ et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k
 
 /* et_attention with the sequence start table of et_sequence_starts handed in (seq_start; one table serves
  * every layer of a batch, as in et_layer_with_prepared), so that the call is the attention kernel alone.  With
- * seq_start NULL the table is built into seq_start_scratch (et_seq_workspace_bytes(B) bytes) first, which is what
- * et_attention does.  No
+ * seq_start NULL the table is built into seq_start_scratch first, which is what et_attention does.  seq_table_bytes is
+ * the size of whichever of the two buffers is used: ET_WORKSPACE_TOO_SMALL below et_seq_workspace_bytes(B).  No
  * counterpart in the reference, whose attention works on padded buffers. */
 et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v,
                                    int qkv_layout, int packed_ld, const void* attr_mask, void* dst,
                                    const int32_t* valid_word_num_dev, int batch_size, int seq_len, int head_num,
                                    int size_per_head, const int32_t* batch_idx, const int32_t* word_idx,
-                                   const int32_t* seq_start, int32_t* seq_start_scratch, void* stream);
+                                   const int32_t* seq_start, int32_t* seq_start_scratch, size_t seq_table_bytes,
+                                   void* stream);
 
 /* Replaces the cublasGemmEx call sites (tf_op/bert_transformer_op.cu.cc:110-141, 200-240):
  * C[m,n] = A[m,k] . B[k,n], all row-major, alpha = 1, beta = 0, fp32 accumulation, C of dtype.

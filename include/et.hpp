@@ -79,7 +79,7 @@ class Encoder {
           bool prepare = true)
       : handle_(device), dtype_(dtype), heads_(head_num), d_(size_per_head), layers_(std::move(layers)) {
     prepared_.assign(layers_.size(),
-                     et_layer_prepared{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0});
+                     et_layer_prepared{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0});
     if (!prepare || dtype != ET_FP16) return;
     check_hip(hipSetDevice(device), "hipSetDevice");
     const size_t H = (size_t)head_num * size_per_head;
@@ -146,7 +146,8 @@ class Encoder {
       pending = true;
     }
     // one sequence start table serves every layer of the batch
-    check(et_sequence_starts(handle_.get(), batch_idx, count, batch, seq_len, starts, stream), handle_.get());
+    check(et_sequence_starts(handle_.get(), batch_idx, count, batch, seq_len, starts, et_seq_workspace_bytes(batch), stream),
+          handle_.get());
     const char* x = act;
     for (size_t l = 0; l < layers_.size(); ++l) {
       if (l == 1 && pending) {       // the first layer is in the queue: waiting here leaves the GPU with work
@@ -157,6 +158,7 @@ class Encoder {
       char* y = act + (1 + (l & 1)) * rows * H * e;
       et_layer_prepared prep = prepared_[l];
       prep.seq_start = starts;
+      prep.seq_start_bytes = et_seq_workspace_bytes(batch);
       check(et_layer_with_prepared(handle_.get(), dtype_, &layers_[l], &prep, x, x, attr_mask, count, batch_idx, word_idx, y,
                                    batch, seq_len, seq_len, heads_, d_, host_count, ws, ws_.capacity(), stream),
             handle_.get());

@@ -309,6 +309,23 @@ def test_error_paths():
     assert st == 1 and b"alias" in lib.et_last_error(h)
     with pytest.raises(TypeError):
         ops.effective_transformer_input(x.to(torch.bfloat16), mask, wl.B, wl.S, wl.S, wl.heads, wl.d)
+    # a sequence table of B + 1 words (2 B + 1 are needed) is refused wherever one is handed in or asked for
+    small = torch.zeros(wl.B + 1, dtype=torch.int32, device="cuda")
+    nsmall = small.numel() * 4
+    st = lib.et_sequence_starts(h, bidx.data_ptr(), vwn.data_ptr(), wl.B, wl.S, small.data_ptr(), nsmall, None)
+    assert st == 2 and b"et_seq_workspace_bytes" in lib.et_last_error(h)
+    prep = _lib.LayerPrepared()
+    prep.seq_start, prep.seq_start_bytes = small.data_ptr(), nsmall
+    ws = torch.empty(lib.et_layer_workspace_bytes(0, wl.B, wl.S, wl.heads, wl.d), dtype=torch.uint8, device="cuda")
+    st = lib.et_layer_with_prepared(h, 0, C.byref(lw.struct), C.byref(prep), to.data_ptr(), to.data_ptr(), attr.data_ptr(),
+                                    vwn.data_ptr(), bidx.data_ptr(), widx.data_ptr(), out.data_ptr(), wl.B, wl.S, wl.S,
+                                    wl.heads, wl.d, -1, ws.data_ptr(), ws.numel(), None)
+    assert st == 2 and b"seq_start" in lib.et_last_error(h)
+    qkv = torch.zeros(wl.B * wl.S, 3 * wl.H, device="cuda")
+    st = lib.et_attention_with_starts(h, 0, qkv.data_ptr(), qkv.data_ptr(), qkv.data_ptr(), 1, 3 * wl.H, attr.data_ptr(),
+                                      out.data_ptr(), vwn.data_ptr(), wl.B, wl.S, wl.heads, wl.d, bidx.data_ptr(),
+                                      widx.data_ptr(), small.data_ptr(), None, nsmall, None)
+    assert st == 2 and b"et_seq_workspace_bytes" in lib.et_last_error(h)
     torch.cuda.synchronize()
 
 

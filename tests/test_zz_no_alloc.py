@@ -69,3 +69,82 @@ def test_static_scratch_input_rejects_sizes_beyond_its_scratch():
     assert st == 3 and b"1048576" in lib.et_last_error(h)
     st = lib.et_input_static(h, _lib.ET_FP16, p, p, p, p, p, None, 4, 4, 1, 64, None)
     assert st == 1
+
+
+def _static_call(lib, h, x, mask, stream):
+    """One et_input_static call on `stream` (a torch stream or None) into fresh outputs; returns (status, outputs)."""
+    B, S = mask.shape
+    to = torch.full_like(x, -7.0)
+    vwn = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+    bidx = torch.full_like(mask, -1)
+    widx = torch.full_like(mask, -1)
+    if stream is not None:
+        stream.wait_stream(torch.cuda.current_stream())      # the fills above run on torch's current stream
+    st = lib.et_input_static(h, _lib.ET_FP16, x.data_ptr(), mask.data_ptr(), to.data_ptr(), vwn.data_ptr(),
+                             bidx.data_ptr(), widx.data_ptr(), B, S, 1, x.shape[-1],
+                             None if stream is None else C.c_void_p(stream.cuda_stream))
+    return st, (to, vwn, bidx, widx)
+
+
+def _big_batch(seed, B=2300, S=64, H=64):
+    rng = np.random.RandomState(seed)
+    lens = rng.randint(0, S + 1, size=B)
+    mask_np = (np.arange(S)[None, :] < lens[:, None]).astype(np.int32)
+    x = torch.from_numpy(rng.randn(B, S, H).astype(np.float32)).cuda().half()
+    return x, torch.from_numpy(mask_np).cuda(), mask_np
+
+
+def test_static_scratch_slots_belong_to_handles():
+    """Every handle owns a slot of the static scratch, so two handles on two streams may overlap; a ninth live handle
+    on the GPU has no slot; the calls of one handle are refused on a second stream while the first still has work."""
+    lib = _lib.load()
+    ops.handle(torch.device("cuda", 0))                  # the package's own handle holds one slot
+    handles = []
+    try:
+        for _ in range(8):
+            h = C.c_void_p()
+            _lib.check(lib.et_create(C.byref(h), 0), None)
+            handles.append(h)
+        x, mask, mask_np = _big_batch(21)
+        x2, mask2, mask2_np = _big_batch(22, B=2200)
+        torch.cuda.synchronize()
+        # the ninth live handle of the GPU got no slot
+        st, _ = _static_call(lib, handles[7], x, mask, None)
+        assert st == 3 and b"slot" in lib.et_last_error(handles[7])
+        # two handles, two streams, queued back to back: each scans through its own slot (144 / 138 tile totals)
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        for _ in range(3):
+            st1, r1 = _static_call(lib, handles[0], x, mask, s1)
+            st2, r2 = _static_call(lib, handles[1], x2, mask2, s2)
+            assert st1 == 0 and st2 == 0
+        torch.cuda.synchronize()
+        for (to, vwn, bidx, widx), m_np, xin in ((r1, mask_np, x), (r2, mask2_np, x2)):
+            pos = np.flatnonzero(m_np.ravel())
+            T = len(pos)
+            S = m_np.shape[1]
+            assert int(vwn.item()) == T
+            assert np.array_equal(bidx.ravel()[:T].cpu().numpy(), pos // S)
+            assert np.array_equal(widx.ravel()[:T].cpu().numpy(), pos % S)
+            assert torch.equal(to.reshape(-1, to.shape[-1])[:T], xin.reshape(-1, to.shape[-1])[torch.from_numpy(pos).cuda()])
+        # one handle, second stream while the first is still busy (a 50 ms sleep queued behind the call): refused
+        st, _ = _static_call(lib, handles[0], x, mask, s1)
+        assert st == 0
+        with torch.cuda.stream(s1):
+            torch.cuda._sleep(int(50e-3 * 2.0e9))
+        st, _ = _static_call(lib, handles[0], x, mask, s2)
+        assert st == 1 and b"in flight" in lib.et_last_error(handles[0])
+        s1.synchronize()
+        st, _ = _static_call(lib, handles[0], x, mask, s2)      # the first stream is idle now: accepted
+        assert st == 0
+        torch.cuda.synchronize()
+        # a destroyed handle gives its slot back
+        _lib.check(lib.et_destroy(handles.pop(0)), None)
+        h = C.c_void_p()
+        _lib.check(lib.et_create(C.byref(h), 0), None)
+        handles.append(h)
+        st, _ = _static_call(lib, h, x, mask, None)
+        assert st == 0
+        torch.cuda.synchronize()
+    finally:
+        for h in handles:
+            lib.et_destroy(h)
