@@ -216,10 +216,12 @@ __device__ __forceinline__ float xor_lanes_16_32_sum(float v) {
   return a + b;
 }
 
-// CPT = 16-byte chunks of one matrix a thread moves per head (ceil(seq rows * chunks per row / 256)).
+// WAVES: wavefronts per workgroup, 4 or 8 (8 for the 128-key fp16 kernel: a query tile per wavefront instead of two, so
+// a head of a long sequence, whose workgroup is the kernel's critical path when few sequences are long, takes half the
+// time).  CPT = 16-byte chunks of one matrix a thread moves per head (ceil(seq rows * chunks per row / threads)).
 // PF: keep the next head's Q/K/V chunks in registers while the current head is computed.
-template <typename T, int NKT, int CPT, bool PF>
-__global__ __launch_bounds__(kAttnThreads) void attention_kernel(
+template <typename T, int NKT, int WAVES, int CPT, bool PF>
+__global__ __launch_bounds__(WAVES * kWave, WAVES == 8 ? 4 : 1) void attention_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, int heads_per_wg, float scaler) {
@@ -231,7 +233,8 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   constexpr int kVR = AttnCfg<_Float16>::kVStride;   // fp16: stride of the row-major V tile
   constexpr int kSp = Sm::kSp;
   constexpr int kCpr = kD / C::kElems;       // 16-byte chunks per head row
-  constexpr int QPW = NKT > 4 ? NKT / 4 : 1; // query tiles per wavefront
+  constexpr int kThreads = WAVES * kWave;
+  constexpr int QPW = NKT > WAVES ? NKT / WAVES : 1;   // query tiles per wavefront
   typedef T mask4 __attribute__((ext_vector_type(4)));
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -260,7 +263,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   int my_t[CPT], my_pos[CPT], my_c[CPT];
 #pragma unroll
   for (int k = 0; k < CPT; ++k) {
-    const int i = threadIdx.x + k * kAttnThreads;
+    const int i = threadIdx.x + k * kThreads;
     const int tt = i / kCpr;
     my_c[k] = i - tt * kCpr;
     my_t[k] = tt < len ? t0 + tt : -1;
@@ -271,7 +274,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   const bool vec_mask = (seq_len & 3) == 0;
 #pragma unroll
   for (int qi = 0; qi < QPW; ++qi) {
-    const int q = (wave + qi * kAttnWaves) * 16 + l16;
+    const int q = (wave + qi * WAVES) * 16 + l16;
     const T* mrow = attr_mask + ((size_t)b * seq_len + min(q, seq_len - 1)) * seq_len;
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) {
@@ -320,7 +323,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
         mreg[qi][kt][r] = kt * 16 + g * 4 + r < seq_len ? (T)((1.0f - (float)mreg[qi][kt][r]) * -10000.0f) : (T)-INFINITY;
 
   // ---- position table, then zero the key / value slots that hold no token (once: heads only overwrite tokens) ----
-  for (int i = threadIdx.x; i < kSp; i += kAttnThreads) tok_of_pos[i] = -1;
+  for (int i = threadIdx.x; i < kSp; i += kThreads) tok_of_pos[i] = -1;
   __syncthreads();
 #pragma unroll
   for (int k = 0; k < CPT; ++k)
@@ -330,7 +333,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
     // the fp16 P.V contraction runs over pairs of key tiles, so an odd tile count drags one more tile of Vt in
     const int rows = min(kSp, ((n_tiles + 1) / 2) * 32);
     // K: row `pos` (kQS elements), Vt: column `pos` of every feature row
-    for (int i = threadIdx.x; i < rows * (kD / 2); i += kAttnThreads) {
+    for (int i = threadIdx.x; i < rows * (kD / 2); i += kThreads) {
       const int pos = i / (kD / 2), w = i - pos * (kD / 2);
       if (tok_of_pos[pos] < 0) {
         if (sizeof(T) == 2) {
@@ -349,7 +352,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
   T* out_row[QPW];
 #pragma unroll
   for (int qi = 0; qi < QPW; ++qi) {
-    const int qt = wave + qi * kAttnWaves;
+    const int qt = wave + qi * WAVES;
     const int tq = qt < n_tiles ? tok_of_pos[qt * 16 + l16] : -1;
     out_row[qi] = tq >= 0 ? dst + (size_t)tq * H + g * (sizeof(T) == 2 ? 16 : 4) : nullptr;
   }
@@ -377,7 +380,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_kernel(
 
 #pragma unroll
     for (int qi = 0; qi < QPW; ++qi) {
-      const int qt = wave + qi * kAttnWaves;
+      const int qt = wave + qi * WAVES;
       if (qt >= n_tiles) break;               // wave-uniform
       const int q = qt * 16 + l16;            // this lane's query position
       float s[NKT][4];
@@ -538,9 +541,13 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
                       float scaler, hipStream_t stream) {
   using Sm = AttnSmem<T, NKT>;
   constexpr int kCpr = kD * (int)sizeof(T) / 16;
-  constexpr int CPT = (NKT * 16 * kCpr + kAttnThreads - 1) / kAttnThreads;
+  // 8 wavefronts where a wavefront of four would serve two query tiles (fp16; the fp32 kernel has no registers to spare
+  // for two workgroups' worth of wavefronts on a CU either way)
+  constexpr int WAVES = (NKT > 4 && sizeof(T) == 2) ? 8 : 4;
+  constexpr int kThreads = WAVES * kWave;
+  constexpr int CPT = (NKT * 16 * kCpr + kThreads - 1) / kThreads;
   constexpr bool PF = CPT <= 4;                // more than 4 chunks x 3 matrices in flight would not fit the registers
-  auto kern = attention_kernel<T, NKT, CPT, PF>;
+  auto kern = attention_kernel<T, NKT, WAVES, CPT, PF>;
   allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)Sm::kBytes);
   // A workgroup serves several heads of one sequence: mask rows, positions and zero fill are shared by them, and the
   // chain of dependent loads a workgroup starts with (sequence start, positions, rows) is paid once.  Up to 6 heads
@@ -553,7 +560,7 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
       break;
     }
   dim3 grid((heads + hpw - 1) / hpw, batch);
-  kern<<<grid, kAttnThreads, Sm::kBytes, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
+  kern<<<grid, kThreads, Sm::kBytes, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
                                                    (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch, seq_len,
                                                    heads, hpw, scaler);
 }
