@@ -22,7 +22,7 @@ OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libet_hip.so")
 EXAMPLE = os.path.join(LIBDIR, "et_encoder_example")      # C++ host sample (csrc/encoder_example.cpp)
 
-SOURCES = ["input_output.hip", "row_kernels.hip", "attention.hip", "gemm.hip", "calibrate.hip", "et_api.cpp"]
+SOURCES = ["input_output.hip", "row_kernels.hip", "attention.hip", "gemm.hip", "generic.hip", "calibrate.hip", "et_api.cpp"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

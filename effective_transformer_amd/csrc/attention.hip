@@ -1729,7 +1729,7 @@ template <typename T>
 __global__ __launch_bounds__(kAttnThreads) void attention_generic_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
-    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, int d, float scaler) {
+    const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, int d, int rows_16b, float scaler) {
   using C = Chunk16<T>;
   using V16 = typename C::vec;
   constexpr int kPerLane = kGenMaxSeq / kWave;             // keys per lane
@@ -1776,10 +1776,14 @@ __global__ __launch_bounds__(kAttnThreads) void attention_generic_kernel(
       float dot = 0.f;
       if (tk >= 0) {
         const T* krow = k_src + src_off(tk, key);
-        for (int c = 0; c < d; c += C::kElems) {
-          const V16 kv = *reinterpret_cast<const V16*>(krow + c);
+        if (rows_16b) {                                    // wave-uniform: head rows of whole, aligned 16-byte pieces
+          for (int c = 0; c < d; c += C::kElems) {
+            const V16 kv = *reinterpret_cast<const V16*>(krow + c);
 #pragma unroll
-          for (int j = 0; j < C::kElems; ++j) dot += qrow[wave][c + j] * (float)kv[j];
+            for (int j = 0; j < C::kElems; ++j) dot += qrow[wave][c + j] * (float)kv[j];
+          }
+        } else {
+          for (int c = 0; c < d; ++c) dot += qrow[wave][c] * (float)krow[c];
         }
       }
       const float sc = (float)(T)dot;                      // the score is stored in the element type
@@ -1828,6 +1832,14 @@ __global__ __launch_bounds__(kAttnThreads) void attention_generic_kernel(
   }
 }
 
+// true when every head row of Q, K and V starts on a 16-byte boundary and is a whole number of 16-byte pieces (what the
+// MFMA kernels and the vector loads of the generic one assume)
+template <typename T>
+bool head_rows_16b(const void* q, const void* k, const void* v, int layout, int packed_ld, int d) {
+  const bool ptrs = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) & 15) == 0;
+  return ptrs && ((size_t)d * sizeof(T)) % 16 == 0 && (layout != 1 || ((size_t)packed_ld * sizeof(T)) % 16 == 0);
+}
+
 template <typename T>
 void attention_generic_launch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                               void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len,
@@ -1835,14 +1847,16 @@ void attention_generic_launch(const void* q, const void* k, const void* v, int l
   dim3 grid((seq_len + kAttnWaves - 1) / kAttnWaves, heads, batch);
   attention_generic_kernel<T><<<grid, kAttnThreads, 0, stream>>>((const T*)q, (const T*)k, (const T*)v, layout, packed_ld,
                                                                  (const T*)attr_mask, (T*)dst, seq_start, word_idx, batch,
-                                                                 seq_len, heads, d, scaler);
+                                                                 seq_len, heads, d,
+                                                                 head_rows_16b<T>(q, k, v, layout, packed_ld, d) ? 1 : 0,
+                                                                 scaler);
 }
 
 template <typename T>
 void attention_dispatch(const void* q, const void* k, const void* v, int layout, int packed_ld, const void* attr_mask,
                         void* dst, const int32_t* seq_start, const int32_t* word_idx, int batch, int seq_len, int heads,
                         int d, float scaler, hipStream_t stream) {
-  if (d != kD)
+  if (d != kD || !head_rows_16b<T>(q, k, v, layout, packed_ld, d))
     attention_generic_launch<T>(q, k, v, layout, packed_ld, attr_mask, dst, seq_start, word_idx, batch, seq_len, heads, d,
                                 scaler, stream);
   else if (seq_len > 512)
@@ -1879,6 +1893,11 @@ void attention_dispatch(const void* q, const void* k, const void* v, int layout,
 void launch_qkv_bias_pad(DType t, const void* Q, const void* bQ, const void* K, const void* bK, const void* V,
                          const void* bV, void* q_buf, void* k_buf, void* v_buf, const int32_t* seq_start,
                          const int32_t* word_idx, int batch, int seq_len, int heads, int d, hipStream_t stream) {
+  if (((size_t)d * elem_size(t)) % 16 != 0) {      // head rows that are no whole number of 16-byte pieces
+    launch_qkv_bias_pad_generic(t, Q, bQ, K, bK, V, bV, q_buf, k_buf, v_buf, seq_start, word_idx, batch, seq_len, heads,
+                                d, stream);
+    return;
+  }
   dim3 grid(batch, 3);
   if (t == DType::F32)
     qkv_bias_pad_kernel<float><<<grid, kPadThreads, 0, stream>>>(
@@ -1907,6 +1926,10 @@ void launch_transpose_rm_padding(DType t, const void* src, void* dst, const int3
                                  int batch, int seq_len, int heads, int d, const int32_t* batch_idx,
                                  const int32_t* word_idx, hipStream_t stream) {
   (void)batch;
+  if (((size_t)d * elem_size(t)) % 16 != 0) {
+    launch_transpose_rm_padding_generic(t, src, dst, rows_dev, rows_bound, seq_len, heads, d, batch_idx, word_idx, stream);
+    return;
+  }
   const int cpd = (int)((size_t)d * elem_size(t) / 16);
   const long total = (long)rows_bound * heads * cpd;
   const int grid = (int)((total + 255) / 256);
@@ -1921,8 +1944,8 @@ void launch_transpose_rm_padding(DType t, const void* src, void* dst, const int3
 }
 
 bool attention_supported(DType t, int seq_len, int d) {
-  // rows of a head are moved in 16-byte pieces
-  return d >= 1 && d <= kGenMaxD && ((size_t)d * elem_size(t)) % 16 == 0 && seq_len >= 1 && seq_len <= kGenMaxSeq;
+  (void)t;
+  return d >= 1 && d <= kGenMaxD && seq_len >= 1 && seq_len <= kGenMaxSeq;
 }
 
 void launch_attention(DType t, const void* q, const void* k, const void* v, int layout, int packed_ld,

@@ -318,8 +318,7 @@ et_status et_input(et_handle h, et_dtype dtype, const void* from_tensor, const i
   if (workspace_bytes < et_input_workspace_bytes(batch_size, seq_len))
     return fail(h, ET_WORKSPACE_TOO_SMALL, "et_input needs et_input_workspace_bytes(batch_size, seq_len)");
   const size_t row_bytes = (size_t)head_num * size_per_head * et::elem_size(to_dt(dtype));
-  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
-  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+  if (et::move_chunks(batch_size * seq_len, (int)row_bytes) >= (1ull << 31))
     return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
   hipStream_t st = (hipStream_t)stream;
   et::launch_scan_index(mask, batch_size * seq_len, nullptr, batch_idx, word_idx, valid_word_num_dev, seq_len,
@@ -353,8 +352,7 @@ et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, 
     return fail(h, ET_UNSUPPORTED,
                 "this handle holds no slot of the static scratch (at most 8 live handles per GPU do); use et_input");
   const size_t row_bytes = (size_t)head_num * size_per_head * et::elem_size(to_dt(dtype));
-  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
-  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+  if (et::move_chunks(batch_size * seq_len, (int)row_bytes) >= (1ull << 31))
     return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
   int32_t* scratch_dev = h->device < kMaxDevices ? static_scratch_ptr[h->device] : nullptr;
   if (!scratch_dev) return fail(h, ET_RUNTIME_ERROR, "no static scratch on this device");
@@ -406,8 +404,8 @@ et_status et_embedding_input(et_handle h, et_dtype dtype, const et_embedding_wei
   if (workspace_bytes < et_input_workspace_bytes(batch_size, seq_len))
     return fail(h, ET_WORKSPACE_TOO_SMALL, "et_embedding_input needs et_input_workspace_bytes(batch_size, seq_len)");
   const int H = head_num * size_per_head;
-  if (!et::bias_residual_layernorm_supported(to_dt(dtype), H))
-    return fail(h, ET_UNSUPPORTED, "hidden size not supported by the LayerNorm kernel");
+  if (!et::layernorm_row_in_registers(to_dt(dtype), H))
+    return fail(h, ET_UNSUPPORTED, "hidden size not supported by the embedding kernel (even, at most 4096)");
   hipStream_t st = (hipStream_t)stream;
   et::launch_scan_index(mask, batch_size * seq_len, nullptr, batch_idx, word_idx, valid_word_num_dev, seq_len,
                         (int32_t*)workspace, st);
@@ -476,7 +474,7 @@ et_status et_layer_with_prepared(et_handle h, et_dtype dtype, const et_layer_wei
   const et::DType dt = to_dt(dtype);
   if ((s = batch_fits_grid(h, B)) != ET_OK) return s;
   if (!et::attention_supported(dt, S, size_per_head))
-    return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 in multiples of 16 bytes and seq_len <= 1024");
+    return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 and seq_len <= 1024");
   if (!et::gemm_supported(dt, H, H, 3) || !et::gemm_supported(dt, F, H, 1) || !et::gemm_supported(dt, H, F, 1))
     return fail(h, ET_UNSUPPORTED, "hidden size not supported by the GEMM kernels");
   if ((uint64_t)B * S * F * et::elem_size(dt) > 0xffffffffull)
@@ -652,8 +650,7 @@ et_status et_compress(et_handle h, et_dtype dtype, const void* from_tensor, cons
   if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && mask && prefix_sum && to_tensor && batch_idx && word_idx, "null tensor pointer");
   const size_t row_bytes = (size_t)hidden_dim * et::elem_size(to_dt(dtype));
-  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
-  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+  if (et::move_chunks(batch_size * seq_len, (int)row_bytes) >= (1ull << 31))
     return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
   hipStream_t st = (hipStream_t)stream;
   et::launch_index_from_prefix(mask, prefix_sum, batch_idx, word_idx, batch_size, seq_len, st);
@@ -672,8 +669,7 @@ et_status et_restore(et_handle h, et_dtype dtype, void* to_tensor, const void* f
   if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
   const size_t row_bytes = (size_t)hidden_dim * et::elem_size(to_dt(dtype));
-  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
-  if ((size_t)batch_size * seq_len * (row_bytes / 16) >= (1ull << 31))
+  if (et::move_chunks(batch_size * seq_len, (int)row_bytes) >= (1ull << 31))
     return fail(h, ET_UNSUPPORTED, "tensor too large for one launch");
   et::launch_restore_rows(to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size, seq_len,
                           (int)row_bytes, (hipStream_t)stream);
@@ -726,8 +722,7 @@ et_status et_add_qkv_bias_padding(et_handle h, et_dtype dtype, const void* Q, co
   ET_REQUIRE(h, workspace != nullptr, "null workspace");
   if (workspace_bytes < et_seq_workspace_bytes(batch_size))
     return fail(h, ET_WORKSPACE_TOO_SMALL, "needs et_seq_workspace_bytes(batch_size)");
-  if (((size_t)size_per_head * et::elem_size(to_dt(dtype))) % 16 != 0 || seq_len > 1024)
-    return fail(h, ET_UNSUPPORTED, "size_per_head bytes must be a multiple of 16 and seq_len <= 1024");
+  if (seq_len > 1024) return fail(h, ET_UNSUPPORTED, "seq_len <= 1024");
   hipStream_t st = (hipStream_t)stream;
   et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, (int32_t*)workspace, st);
   et::launch_qkv_bias_pad(to_dt(dtype), Q, bias_Q, K, bias_K, V, bias_V, q_buf, k_buf, v_buf, (int32_t*)workspace,
@@ -757,8 +752,6 @@ et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, 
   ET_REQUIRE(h, dtype_ok(dtype), "dtype must be ET_FP32 or ET_FP16");
   if ((s = dims_ok(h, batch_size, seq_len, head_num, size_per_head)) != ET_OK) return s;
   ET_REQUIRE(h, src && dst && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
-  if (((size_t)size_per_head * et::elem_size(to_dt(dtype))) % 16 != 0)
-    return fail(h, ET_UNSUPPORTED, "size_per_head bytes must be a multiple of 16");
   et::launch_transpose_rm_padding(to_dt(dtype), src, dst, valid_word_num_dev, batch_size * seq_len, batch_size,
                                   seq_len, head_num, size_per_head, batch_idx, word_idx, (hipStream_t)stream);
   return check_launch(h, "transpose + remove padding");
@@ -797,9 +790,7 @@ et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, c
     return fail(h, ET_WORKSPACE_TOO_SMALL, "the sequence table needs et_seq_workspace_bytes(batch_size)");
   if ((s = batch_fits_grid(h, batch_size)) != ET_OK) return s;
   if (!et::attention_supported(to_dt(dtype), seq_len, size_per_head))
-    return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 in multiples of 16 bytes and seq_len <= 1024");
-  if (qkv_layout == 1 && ((size_t)packed_ld * et::elem_size(to_dt(dtype))) % 16 != 0)
-    return fail(h, ET_UNSUPPORTED, "packed_ld bytes must be a multiple of 16");
+    return fail(h, ET_UNSUPPORTED, "attention needs size_per_head <= 256 and seq_len <= 1024");
   hipStream_t st = (hipStream_t)stream;
   if (!seq_start) {
     et::launch_seq_start(batch_idx, valid_word_num_dev, batch_size * seq_len, batch_size, seq_start_scratch, st);
@@ -822,8 +813,7 @@ et_status gemm_impl(et_handle h, et_dtype dtype, const void* A, const void* B, v
   ET_REQUIRE(h, !gelu || bias, "null bias");
   ET_REQUIRE(h, m >= 0 && n >= 1 && k >= 1, "bad dimensions");
   if (!et::gemm_supported(to_dt(dtype), n, k, 1))
-    return fail(h, ET_UNSUPPORTED, dtype == ET_FP16 ? "fp16 GEMM needs k % 32 == 0 and n % 8 == 0"
-                                                     : "fp32 GEMM needs k % 16 == 0 and n % 4 == 0");
+    return fail(h, ET_UNSUPPORTED, "GEMM dimensions out of range");
   if ((uint64_t)m * k * et::elem_size(to_dt(dtype)) > 0xffffffffull)
     return fail(h, ET_UNSUPPORTED, "A larger than 4 GB");
   if (m == 0) return ET_OK;

@@ -1427,9 +1427,18 @@ __global__ __launch_bounds__(256) void layer_prologue_kernel(TransposeArgs args)
 
 }  // namespace
 
+namespace {
+// what the MFMA kernels take
+bool gemm_tiled(DType t, int n, int k) {
+  if (t == DType::F16) return k % kHBK == 0 && n % 8 == 0 && n >= 8;
+  return k % kFBK == 0 && n % 4 == 0 && (uint64_t)k * (uint64_t)n * 4u < 0x80000000ull;
+}
+}  // namespace
+
 bool gemm_takes_transposed_b(DType t, int m_bound, int ldc, int n, int k, int groups) {
   (void)m_bound; (void)ldc;
-  return t == DType::F16 && gemm_supported(t, n, k, groups) && k % 64 == 0 && (uint64_t)k * 256u * 2u < 0x80000000ull;
+  return t == DType::F16 && gemm_supported(t, n, k, groups) && gemm_tiled(t, n, k) && k % 64 == 0 &&
+         (uint64_t)k * 256u * 2u < 0x80000000ull;
 }
 
 bool gemm_blocked_handover(DType t, int m_bound, int wide, int narrow) {
@@ -1465,14 +1474,17 @@ void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, con
 }
 
 bool gemm_supported(DType t, int n, int k, int groups) {
-  if (groups < 1 || groups > 3 || n <= 0 || k <= 0) return false;
-  if (t == DType::F16) return k % kHBK == 0 && n % 8 == 0 && n >= 8;
-  return k % kFBK == 0 && n % 4 == 0 && (uint64_t)k * (uint64_t)n * 4u < 0x80000000ull;
+  (void)t;
+  return groups >= 1 && groups <= 3 && n > 0 && k > 0;
 }
 
 void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k, const int32_t* rows_dev,
                  hipStream_t stream) {
   if (m_bound <= 0) return;
+  if (!gemm_tiled(t, n, k)) {
+    launch_gemm_generic(t, g, C, ldc, m_bound, n, k, rows_dev, stream);
+    return;
+  }
   GemmArgs a;
   for (int i = 0; i < 3; ++i) {
     a.A[i] = i < g.groups ? g.A[i] : nullptr;

@@ -135,9 +135,12 @@ __global__ __launch_bounds__(256) void index_from_prefix_kernel(const int32_t* _
 constexpr int kMoveThreads = 256;
 constexpr int kMoveUnroll = 8;
 
-// Gather of packed rows: flattened over (packed row, 16-byte chunk).
+// Gather of packed rows: flattened over (packed row, chunk).  CH = the widest piece the row is a whole number of: 16
+// bytes for every hidden size a BERT model has; 4 or 2 bytes for the others (the reference moves single elements,
+// cuda/cuda_kernels.cu:278-384).
+template <typename CH>
 __global__ __launch_bounds__(kMoveThreads) void compress_rows_kernel(
-    const u32x4* __restrict__ from, u32x4* __restrict__ to, const int32_t* __restrict__ batch_idx,
+    const CH* __restrict__ from, CH* __restrict__ to, const int32_t* __restrict__ batch_idx,
     const int32_t* __restrict__ word_idx, const int32_t* __restrict__ rows_dev, const int32_t* __restrict__ prefix,
     const int32_t* __restrict__ mask, int n_pos, int seq_len, fastdiv cpr) {
   int T;
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(kMoveThreads) void compress_rows_kernel(
     bi[u] = batch_idx[row[u]];
     wi[u] = word_idx[row[u]];
   }
-  u32x4 val[kMoveUnroll];
+  CH val[kMoveUnroll];
 #pragma unroll
   for (int u = 0; u < kMoveUnroll; ++u) {
     const uint32_t src_row = (uint32_t)bi[u] * (uint32_t)seq_len + (uint32_t)wi[u];
@@ -181,8 +184,9 @@ constexpr int kRestorePos = 32;   // padded positions per workgroup
 // without scratch memory: keys b*S+s are ascending in t, so a 64-way search by one wavefront
 // locates the first packed row at or after the workgroup's first position and the next
 // kRestorePos keys cover everything that can land in the workgroup's window.
+template <typename CH>
 __global__ __launch_bounds__(kMoveThreads) void restore_rows_kernel(
-    u32x4* __restrict__ to, const u32x4* __restrict__ from, const int32_t* __restrict__ batch_idx,
+    CH* __restrict__ to, const CH* __restrict__ from, const int32_t* __restrict__ batch_idx,
     const int32_t* __restrict__ word_idx, const int32_t* __restrict__ rows_dev, int n_pos, int seq_len, int cpr) {
   __shared__ int inv[kRestorePos];
   __shared__ int t0_sh;
@@ -223,11 +227,11 @@ __global__ __launch_bounds__(kMoveThreads) void restore_rows_kernel(
   const int npos = min(kRestorePos, n_pos - p0);
   const int total = npos * cpr;
   for (int i0 = 0; i0 < total; i0 += kMoveThreads * kMoveUnroll) {
-    u32x4 val[kMoveUnroll];
+    CH val[kMoveUnroll];
 #pragma unroll
     for (int u = 0; u < kMoveUnroll; ++u) {
       const int i = i0 + u * kMoveThreads + threadIdx.x;
-      val[u] = u32x4{0u, 0u, 0u, 0u};
+      val[u] = CH{};
       if (i < total) {
         const int r = i / cpr;
         const int c = i - r * cpr;
@@ -332,24 +336,50 @@ void launch_index_from_prefix(const int32_t* mask, const int32_t* prefix, int32_
   index_from_prefix_kernel<<<(n + 255) / 256, 256, 0, stream>>>(mask, prefix, batch_idx, word_idx, n, seq_len);
 }
 
+namespace {
+// the widest chunk a row of row_bytes bytes is a whole number of
+inline int move_chunk_bytes(int row_bytes) { return row_bytes % 16 == 0 ? 16 : (row_bytes % 4 == 0 ? 4 : 2); }
+}  // namespace
+
+size_t move_chunks(int n_pos, int row_bytes) { return (size_t)n_pos * (size_t)(row_bytes / move_chunk_bytes(row_bytes)); }
+
 void launch_compress_rows(const void* from, void* to, const int32_t* batch_idx, const int32_t* word_idx,
                           const int32_t* rows_dev, const int32_t* prefix, const int32_t* mask, int batch, int seq_len,
                           int row_bytes, hipStream_t stream) {
   const int n_pos = batch * seq_len;
-  const uint32_t cpr = (uint32_t)row_bytes / 16u;
+  const int cb = move_chunk_bytes(row_bytes);
+  const uint32_t cpr = (uint32_t)row_bytes / (uint32_t)cb;
   const uint64_t chunks = (uint64_t)n_pos * cpr;
   const uint32_t per_wg = kMoveThreads * kMoveUnroll;
   const uint32_t grid = (uint32_t)((chunks + per_wg - 1) / per_wg);
-  compress_rows_kernel<<<grid, kMoveThreads, 0, stream>>>((const u32x4*)from, (u32x4*)to, batch_idx, word_idx,
-                                                          rows_dev, prefix, mask, n_pos, seq_len, make_fastdiv(cpr));
+  if (cb == 16)
+    compress_rows_kernel<u32x4><<<grid, kMoveThreads, 0, stream>>>((const u32x4*)from, (u32x4*)to, batch_idx, word_idx,
+                                                                   rows_dev, prefix, mask, n_pos, seq_len, make_fastdiv(cpr));
+  else if (cb == 4)
+    compress_rows_kernel<uint32_t><<<grid, kMoveThreads, 0, stream>>>((const uint32_t*)from, (uint32_t*)to, batch_idx,
+                                                                      word_idx, rows_dev, prefix, mask, n_pos, seq_len,
+                                                                      make_fastdiv(cpr));
+  else
+    compress_rows_kernel<uint16_t><<<grid, kMoveThreads, 0, stream>>>((const uint16_t*)from, (uint16_t*)to, batch_idx,
+                                                                      word_idx, rows_dev, prefix, mask, n_pos, seq_len,
+                                                                      make_fastdiv(cpr));
 }
 
 void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
                          const int32_t* rows_dev, int batch, int seq_len, int row_bytes, hipStream_t stream) {
   const int n_pos = batch * seq_len;
   const int grid = (n_pos + kRestorePos - 1) / kRestorePos;
-  restore_rows_kernel<<<grid, kMoveThreads, 0, stream>>>((u32x4*)to, (const u32x4*)from, batch_idx, word_idx, rows_dev,
-                                                         n_pos, seq_len, row_bytes / 16);
+  const int cb = move_chunk_bytes(row_bytes);
+  const int cpr = row_bytes / cb;
+  if (cb == 16)
+    restore_rows_kernel<u32x4><<<grid, kMoveThreads, 0, stream>>>((u32x4*)to, (const u32x4*)from, batch_idx, word_idx,
+                                                                  rows_dev, n_pos, seq_len, cpr);
+  else if (cb == 4)
+    restore_rows_kernel<uint32_t><<<grid, kMoveThreads, 0, stream>>>((uint32_t*)to, (const uint32_t*)from, batch_idx,
+                                                                     word_idx, rows_dev, n_pos, seq_len, cpr);
+  else
+    restore_rows_kernel<uint16_t><<<grid, kMoveThreads, 0, stream>>>((uint16_t*)to, (const uint16_t*)from, batch_idx,
+                                                                     word_idx, rows_dev, n_pos, seq_len, cpr);
 }
 
 void launch_seq_order(int32_t* seq_table, int batch, hipStream_t stream) {

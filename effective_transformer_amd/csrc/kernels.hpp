@@ -34,6 +34,9 @@ void launch_index_from_prefix(const int32_t* mask, const int32_t* prefix, int32_
 void launch_compress_rows(const void* from, void* to, const int32_t* batch_idx, const int32_t* word_idx,
                           const int32_t* rows_dev, const int32_t* prefix, const int32_t* mask,
                           int batch, int seq_len, int row_bytes, hipStream_t stream);
+// Chunks (16, 4 or 2 bytes: the widest piece row_bytes is a whole number of) the two movers below index for n_pos rows;
+// must stay below 2^31.
+size_t move_chunks(int n_pos, int row_bytes);
 // to[B*S rows] = 0 at padding, from[t] at batch_idx[t]*S + word_idx[t]; indices ascending.
 void launch_restore_rows(void* to, const void* from, const int32_t* batch_idx, const int32_t* word_idx,
                          const int32_t* rows_dev, int batch, int seq_len, int row_bytes, hipStream_t stream);
@@ -53,6 +56,8 @@ bool bias_gelu_supported(DType t, int n);
 void launch_bias_gelu(DType t, void* out, const void* bias, int m, int n, const int32_t* rows_dev,
                       hipStream_t stream);
 bool bias_residual_layernorm_supported(DType t, int n);
+// rows the wave-per-row kernels keep in registers (n a multiple of 2 in fp16, up to 4096 elements)
+bool layernorm_row_in_registers(DType t, int n);
 // Regions whose 128-byte lines a kernel requests on its way (pulled into the last-level cache) for a later kernel that
 // would otherwise read them cold.
 struct WarmList {
@@ -116,6 +121,8 @@ struct GemmGroups {
   // stores are the better choice when C would only push the weights and the A rows out of that cache.
   bool c_cached = false;
 };
+// any n, k >= 1 (the MFMA kernels need k % 32 == 0, n % 8 == 0 in fp16 and k % 16 == 0, n % 4 == 0 in fp32; other
+// shapes run the element-wise kernel of generic.hip)
 bool gemm_supported(DType t, int n, int k, int groups);
 // True when both C = A.B1 ([m, wide] from k = narrow) and the product that consumes it (k = wide, n = narrow) run the
 // persistent k-contiguous kernel, given k-contiguous copies of both weights.
@@ -145,6 +152,22 @@ struct SeqStartJob {
 void launch_transpose_weights(const TransposeJobs& jobs, hipStream_t stream, const SeqStartJob* seq = nullptr);
 void launch_gemm(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k,
                  const int32_t* rows_dev, hipStream_t stream);
+
+// ---- generic.hip: element-wise kernels for the shapes the tuned kernels do not take ------------------------------
+// (rows or head rows that are no whole number of 16-byte pieces, GEMM k / n the MFMA tiles cannot take); the launchers
+// above fall back to them by themselves.
+void launch_gemm_generic(DType t, const GemmGroups& g, void* C, int ldc, int m_bound, int n, int k,
+                         const int32_t* rows_dev, hipStream_t stream);
+void launch_bias_gelu_generic(DType t, void* out, const void* bias, int m, int n, const int32_t* rows_dev,
+                              hipStream_t stream);
+void launch_layernorm_generic(DType t, void* out, const void* input, const void* bias, const void* gamma,
+                              const void* beta, int m, int n, const int32_t* rows_dev, float eps, hipStream_t stream);
+void launch_qkv_bias_pad_generic(DType t, const void* Q, const void* bQ, const void* K, const void* bK, const void* V,
+                                 const void* bV, void* q_buf, void* k_buf, void* v_buf, const int32_t* seq_start,
+                                 const int32_t* word_idx, int batch, int seq_len, int heads, int d, hipStream_t stream);
+void launch_transpose_rm_padding_generic(DType t, const void* src, void* dst, const int32_t* rows_dev, int rows_bound,
+                                         int seq_len, int heads, int d, const int32_t* batch_idx,
+                                         const int32_t* word_idx, hipStream_t stream);
 
 // ---- calibrate.hip: measurement aid ---------------------------------------------------------------------
 // One launch of `iters` k-steps of the large fp16 GEMM's inner loop (MFMAs + LDS operand reads, no global memory) on

@@ -376,9 +376,16 @@ void launch_embed_layernorm(DType t, void* out, const int32_t* ids, const int32_
     embed_launch<_Float16>(a, stream);
 }
 
-bool bias_gelu_supported(DType t, int n) { return n > 0 && ((size_t)n * elem_size(t)) % 16 == 0; }
+bool bias_gelu_supported(DType t, int n) {
+  (void)t;
+  return n > 0;
+}
 
 void launch_bias_gelu(DType t, void* out, const void* bias, int m, int n, const int32_t* rows_dev, hipStream_t stream) {
+  if (((size_t)n * elem_size(t)) % 16 != 0) {      // rows that are no whole number of 16-byte pieces
+    launch_bias_gelu_generic(t, out, bias, m, n, rows_dev, stream);
+    return;
+  }
   const int cpr = (int)((size_t)n * elem_size(t) / 16);
   dim3 grid((cpr + kGeluThreads - 1) / kGeluThreads, (m + kGeluRows - 1) / kGeluRows);
   if (t == DType::F32)
@@ -388,10 +395,15 @@ void launch_bias_gelu(DType t, void* out, const void* bias, int m, int n, const 
                                                                   rows_dev);
 }
 
-bool bias_residual_layernorm_supported(DType t, int n) {
+bool layernorm_row_in_registers(DType t, int n) {
   int vec, iters;
   if (n <= 0) return false;
   return t == DType::F32 ? ln_pick<float>(n, vec, iters) : ln_pick<_Float16>(n, vec, iters);
+}
+
+bool bias_residual_layernorm_supported(DType t, int n) {
+  (void)t;
+  return n > 0;
 }
 
 void WarmList::add(const void* region, size_t bytes) {
@@ -408,6 +420,10 @@ void WarmList::add(const void* region, size_t bytes) {
 void launch_bias_residual_layernorm(DType t, void* out, const void* input, const void* bias, const void* gamma,
                                     const void* beta, int m, int n, const int32_t* rows_dev, hipStream_t stream,
                                     const WarmList& warm) {
+  if (!layernorm_row_in_registers(t, n)) {      // odd or very long rows: three passes over memory
+    launch_layernorm_generic(t, out, input, bias, gamma, beta, m, n, rows_dev, 1e-6f, stream);
+    return;
+  }
   if (t == DType::F32)
     ln_launch<float>(out, input, bias, gamma, beta, m, n, rows_dev, stream, warm);
   else

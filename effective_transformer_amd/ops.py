@@ -209,6 +209,10 @@ class LayerWeights:
         transpose by itself."""
         if self.t["attr_kernel_q"].dtype != torch.float16:
             return self
+        # the k-contiguous kernels take k in multiples of 64 and n in multiples of 8; other hidden sizes run the [k][n] kernels
+        hq = self.t["attr_kernel_q"].shape[0]
+        if hq % 64 != 0:
+            return self
         lib = _lib.load()
         dev = self.t["attr_kernel_q"].device
         h = handle(dev)

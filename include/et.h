@@ -126,8 +126,10 @@ et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, 
  * *valid_word_num_dev, so the call never blocks the host (the reference copies T back every
  * layer, :99-101).
  * from_seq_len must equal to_seq_len (tf_op/bert_transformer_op.cc:130-131).  `out` must not
- * alias from_tensor/to_tensor.  Shapes: seq_len <= 1024, batch_size <= 65535, size_per_head <= 256 (see et_attention),
- * hidden size a multiple of 32 (fp16) or 16 (fp32). */
+ * alias from_tensor/to_tensor.  Shapes: seq_len <= 1024, batch_size <= 65535, any size_per_head from 1 to 256 (see
+ * et_attention).  The tuned kernels take head size 64 and hidden sizes in multiples of 32 (fp16) or 16 (fp32); every
+ * other shape runs element-wise kernels with the same arithmetic (the reference's kernels index by element too,
+ * cuda/attention.cu:190-219). */
 et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,
                    const void* from_tensor, const void* to_tensor, const void* attr_mask,
                    const int32_t* valid_word_num_dev, const int32_t* batch_idx, const int32_t* word_idx,
@@ -282,8 +284,8 @@ et_status et_transpose_rm_padding(et_handle h, et_dtype dtype, const void* src, 
  *   qkv_layout 1: q/k/v point into packed token-major rows (row t, column head*d + j) with row
  *                 stride `packed_ld` elements (bias already added).
  *   dst packed [T,heads*d].  workspace: et_seq_workspace_bytes(B).
- * seq_len <= 1024; size_per_head <= 256 with head rows of whole 16-byte pieces.  size_per_head = 64 runs the
- * MFMA kernels, every other head size a slower general kernel with the same arithmetic. */
+ * seq_len <= 1024; size_per_head from 1 to 256.  size_per_head = 64 (head rows on 16-byte boundaries) runs the MFMA
+ * kernels, every other head size a slower general kernel with the same arithmetic. */
 et_status et_attention(et_handle h, et_dtype dtype, const void* q, const void* k, const void* v, int qkv_layout,
                        int packed_ld, const void* attr_mask, void* dst,
                        const int32_t* valid_word_num_dev, int batch_size, int seq_len,
@@ -306,7 +308,8 @@ et_status et_attention_with_starts(et_handle h, et_dtype dtype, const void* q, c
 /* Replaces the cublasGemmEx call sites (tf_op/bert_transformer_op.cu.cc:110-141, 200-240):
  * C[m,n] = A[m,k] . B[k,n], all row-major, alpha = 1, beta = 0, fp32 accumulation, C of dtype.
  * bias (optional, [n]) is added to the rounded product (in the element type, as the reference's
- * following kernel would).  m_dev (optional) bounds the rows on the device. */
+ * following kernel would).  m_dev (optional) bounds the rows on the device.  Any m, n, k: the MFMA kernels take
+ * k % 32 == 0, n % 8 == 0 (fp16) / k % 16 == 0, n % 4 == 0 (fp32), other shapes an element-wise kernel. */
 et_status et_gemm(et_handle h, et_dtype dtype, const void* A, const void* B, void* C, const void* bias,
                   int m, int n, int k, const int32_t* m_dev, void* stream);
 

@@ -80,7 +80,8 @@ class Encoder {
       : handle_(device), dtype_(dtype), heads_(head_num), d_(size_per_head), layers_(std::move(layers)) {
     prepared_.assign(layers_.size(),
                      et_layer_prepared{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0});
-    if (!prepare || dtype != ET_FP16) return;
+    // (the k-contiguous kernels take hidden sizes in multiples of 64; others run on the weights as they are)
+    if (!prepare || dtype != ET_FP16 || ((size_t)head_num * size_per_head) % 64 != 0) return;
     check_hip(hipSetDevice(device), "hipSetDevice");
     const size_t H = (size_t)head_num * size_per_head;
     char* dst = (char*)wt_.reserve(layers_.size() * 12 * H * H * 2);

@@ -295,8 +295,8 @@ def test_error_paths():
     with pytest.raises(_lib.EtError) as e:       # from_seq_len != to_seq_len
         ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S + 1, wl.heads, wl.d)
     assert e.value.status == 1 and "from_seq_len == to_seq_len" in str(e.value)
-    with pytest.raises(_lib.EtError) as e:       # a head row that is not a whole number of 16-byte pieces
-        ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S, wl.heads * 32, wl.d // 32)
+    with pytest.raises(_lib.EtError) as e:       # a head size beyond what the attention kernels hold
+        ops.effective_transformer(to, to, attr, vwn, bidx, widx, lw, wl.B, wl.S, wl.S, 1, 257)
     assert e.value.status == 3
     out = torch.empty_like(to)
     st = lib.et_layer(h, 0, C.byref(lw.struct), to.data_ptr(), to.data_ptr(), attr.data_ptr(), vwn.data_ptr(),

@@ -148,3 +148,42 @@ def test_static_scratch_slots_belong_to_handles():
     finally:
         for h in handles:
             lib.et_destroy(h)
+
+
+def test_static_scratch_input_under_graph_capture():
+    """What the entry point is for: a caller under HIP graph capture.  Captured once on a handle of its own, replayed
+    with several masks (eager work and synchronisations between the replays), every replay against et_input."""
+    lib = _lib.load()
+    h = C.c_void_p()
+    _lib.check(lib.et_create(C.byref(h), 0), None)
+    try:
+        B, S, H = 2200, 64, 64
+        x, mask, _ = _big_batch(31, B=B)
+        to = torch.full_like(x, -7.0)
+        vwn = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+        bidx = torch.full_like(mask, -1)
+        widx = torch.full_like(mask, -1)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            st = lib.et_input_static(h, _lib.ET_FP16, x.data_ptr(), mask.data_ptr(), to.data_ptr(), vwn.data_ptr(),
+                                     bidx.data_ptr(), widx.data_ptr(), B, S, 1, H,
+                                     C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert st == 0, lib.et_last_error(h)
+        hh = ops.handle(torch.device("cuda", 0))
+        for seed in (41, 42, 43):
+            x2, mask2, mask2_np = _big_batch(seed, B=B)
+            x.copy_(x2)
+            mask.copy_(mask2)
+            g.replay()
+            torch.cuda.synchronize()
+            # the same batch through et_input (eager work between the replays)
+            to_ref, n_ref, b_ref, w_ref = ops.effective_transformer_input(x2, mask2, B, S, S, 1, H)
+            torch.cuda.synchronize()
+            T = int(mask2_np.sum())
+            assert int(vwn.item()) == T == int(n_ref.item())
+            assert torch.equal(bidx.ravel()[:T], b_ref.ravel()[:T]) and torch.equal(widx.ravel()[:T], w_ref.ravel()[:T])
+            assert torch.equal(to.reshape(B * S, -1)[:T], to_ref.reshape(B * S, -1)[:T])
+        del g, hh
+    finally:
+        lib.et_destroy(h)
