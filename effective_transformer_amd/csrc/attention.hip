@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void transpose_rm_padding_kernel(
 // ------------------------------------------------------------------------------------------
 // fused attention, size_per_head = 64, seq_len <= 128 (longer sequences: attention_long_kernel below).
 //
-// One workgroup (4 wavefronts) per (sequence, group of up to 4 heads).  What does not depend on the
+// One workgroup (4 wavefronts, 8 at 128 keys in fp16) per (sequence, group of heads).  What does not depend on the
 // head is done once: token positions, the zero fill of key/value slots without a token (so that a
 // mask that attends to a padded key sees the zero score / zero value the reference's padded buffers
 // hold) and the mask rows of each wavefront's queries, which stay in registers.  Per head the K rows
