@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void transpose_rm_padding_kernel(
 // ------------------------------------------------------------------------------------------
 // fused attention, size_per_head = 64, seq_len <= 128 (longer sequences: attention_long_kernel below).
 //
-// One workgroup (4 wavefronts, 8 at 128 keys in fp16) per (sequence, group of heads).  What does not depend on the
+// One workgroup (4 wavefronts) per (sequence, group of heads).  What does not depend on the
 // head is done once: token positions, the zero fill of key/value slots without a token (so that a
 // mask that attends to a padded key sees the zero score / zero value the reference's padded buffers
 // hold) and the mask rows of each wavefront's queries, which stay in registers.  Per head the K rows
@@ -216,12 +216,11 @@ __device__ __forceinline__ float xor_lanes_16_32_sum(float v) {
   return a + b;
 }
 
-// WAVES: wavefronts per workgroup, 4 or 8 (8 for the 128-key fp16 kernel: a query tile per wavefront instead of two, so
-// a head of a long sequence, whose workgroup is the kernel's critical path when few sequences are long, takes half the
-// time).  CPT = 16-byte chunks of one matrix a thread moves per head (ceil(seq rows * chunks per row / threads)).
+// WAVES: wavefronts per workgroup (4; a wavefront serves NKT / WAVES query tiles at 128 keys).  CPT = 16-byte chunks of
+// one matrix a thread moves per head (ceil(seq rows * chunks per row / threads)).
 // PF: keep the next head's Q/K/V chunks in registers while the current head is computed.
 template <typename T, int NKT, int WAVES, int CPT, bool PF>
-__global__ __launch_bounds__(WAVES * kWave, WAVES == 8 ? 4 : 1) void attention_kernel(
+__global__ __launch_bounds__(WAVES * kWave) void attention_kernel(
     const T* __restrict__ q_src, const T* __restrict__ k_src, const T* __restrict__ v_src, int layout, int packed_ld,
     const T* __restrict__ attr_mask, T* __restrict__ dst, const int32_t* __restrict__ seq_start,
     const int32_t* __restrict__ word_idx, int batch, int seq_len, int heads, int heads_per_wg, float scaler) {
@@ -541,9 +540,9 @@ void attention_launch(const void* q, const void* k, const void* v, int layout, i
                       float scaler, hipStream_t stream) {
   using Sm = AttnSmem<T, NKT>;
   constexpr int kCpr = kD * (int)sizeof(T) / 16;
-  // 8 wavefronts where a wavefront of four would serve two query tiles (fp16; the fp32 kernel has no registers to spare
-  // for two workgroups' worth of wavefronts on a CU either way)
-  constexpr int WAVES = (NKT > 4 && sizeof(T) == 2) ? 8 : 4;
+  // Four wavefronts.  Eight at 128 keys in fp16 (one query tile per wavefront, 128 registers, two workgroups per CU)
+  // run the kernel alone 6 % faster on a batch with few long sequences and no faster inside the layer.
+  constexpr int WAVES = 4;
   constexpr int kThreads = WAVES * kWave;
   constexpr int CPT = (NKT * 16 * kCpr + kThreads - 1) / kThreads;
   constexpr bool PF = CPT <= 4;                // more than 4 chunks x 3 matrices in flight would not fit the registers
