@@ -307,6 +307,12 @@ def test_error_paths():
                       bidx.data_ptr(), widx.data_ptr(), to.data_ptr(), wl.B, wl.S, wl.S, wl.heads, wl.d, -1,
                       out.data_ptr(), 1 << 30, None)
     assert st == 1 and b"alias" in lib.et_last_error(h)
+    # one sequence more than the attention grid holds: refused before anything is launched (the declared workspace
+    # size only has to pass the size check)
+    st = lib.et_layer(h, 0, C.byref(lw.struct), to.data_ptr(), to.data_ptr(), attr.data_ptr(), vwn.data_ptr(),
+                      bidx.data_ptr(), widx.data_ptr(), out.data_ptr(), 65536, 1, 1, wl.heads, wl.d, -1,
+                      out.data_ptr(), 1 << 40, None)
+    assert st == 3 and b"65535" in lib.et_last_error(h)
     with pytest.raises(TypeError):
         ops.effective_transformer_input(x.to(torch.bfloat16), mask, wl.B, wl.S, wl.S, wl.heads, wl.d)
     # a sequence table of B + 1 words (2 B + 1 are needed) is refused wherever one is handed in or asked for
@@ -361,6 +367,26 @@ def test_other_head_sizes_and_sequences_beyond_512(dtype, B, S, heads, d):
     w = dict(wl=wl, lens=lens, mask=mask, attr_mask=o.rnd(attr, dtype), x=x, weights=o.make_layer_weights(wl, rng, True))
     got = run_encoder(w)
     _check(got, _oracle(w), mask, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_largest_batch_the_attention_grid_holds(dtype):
+    """65535 sequences (one more is refused, see test_error_paths): a subset of the sequences against the oracle, and the
+    full run reproduces the subset's rows bit for bit."""
+    print("encoder B=65535", dtype, flush=True)
+    B, S, heads, d = 65535, 4, 2, 64
+    wl = o.Workload("wide-batch", 65535, dtype, 1, B, S, heads, d, 4 * heads * d, 0, S + 1)
+    rng = np.random.RandomState(wl.seed)
+    lens, mask, attr = o.make_masks(wl, rng)
+    x = o.rnd(rng.randn(B, S, wl.H), dtype)
+    w = dict(wl=wl, lens=lens, mask=mask, attr_mask=o.rnd(attr, dtype), x=x, weights=o.make_layer_weights(wl, rng, True))
+    full = run_encoder(w)
+    assert np.all(full[~mask.astype(bool)] == 0)
+    idx = np.sort(np.concatenate([np.arange(20), B - 1 - np.arange(20), rng.choice(np.arange(20, B - 20), 40, replace=False)]))
+    sub = subset_workload(w, idx)
+    got_sub = run_encoder(sub)
+    assert np.array_equal(got_sub, full[idx])
+    _check(got_sub, _oracle(sub), sub["mask"], dtype)
 
 
 @pytest.mark.parametrize("seed", range(12))
