@@ -64,7 +64,10 @@ __global__ __launch_bounds__(kCalThreads) void mfma_ceiling_kernel(float* __rest
           a[1 - P][2 * (i - 2) + 1] = *reinterpret_cast<const half8*>(src + ((2 * (i - 2) + 1) & 3) * 2048 + 32);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[P][i], b[P][j], acc[i][j], 0, 0, 0);
+        for (int jj = 0; jj < 4; ++jj) {
+          const int j = (i & 1) ? 3 - jj : jj;       // back and forth, as in the GEMM: one operand changes per MFMA
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[P][i], b[P][j], acc[i][j], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }

