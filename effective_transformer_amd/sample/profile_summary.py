@@ -325,15 +325,16 @@ def cmd_ceiling(paths):
     out.append("`ds_read_b128` refill the other set from LDS, as `gemm_f16_pair_kernel` does, with no global memory traffic, no barrier")
     out.append("and nothing to wait for but the LDS; 4000 k-steps per launch, best of 2 x 5 launches. One row per run (each on a box of")
     out.append("its own):\n")
-    out.append("| run | zero operands TFLOP/s | random halves TFLOP/s | random / 2500 peak | step ms | dominant kernel in the layer | TFLOP/s | of peak | of the rate on random operands |")
+    out.append("| run | zero operands TFLOP/s | random halves TFLOP/s | random / 2500 peak | step ms | dominant kernel in the layer | achieved | of peak | of the rate on random operands |")
     out.append("|---|---|---|---|---|---|---|---|---|")
     for path in paths:
         d = last_json_line(path)
         c, r = d["mfma_ceiling"], d["roofline"]
-        out.append("| %s | %.0f | %.0f | %.3f | %.3f | %s | %.0f | %.3f | %.3f |" % (
+        of_random = r.get("frac_of_sustained_on_random_operands")      # only where the dominant kernel is MFMA-bound
+        out.append("| %s | %.0f | %.0f | %.3f | %.3f | %s | %.0f %s | %.3f | %s |" % (
             d["config"]["workload"].split(":")[0], c["zero_operands_tflops"], c["random_operands_tflops"],
-            c["random_operands_tflops"] / 2500.0, d["ms_per_step"], r["kernel"], r["achieved"], r["frac"],
-            r.get("frac_of_sustained_on_random_operands", float("nan"))))
+            c["random_operands_tflops"] / 2500.0, d["ms_per_step"], r["kernel"], r["achieved"], r["unit"], r["frac"],
+            "%.3f" % of_random if of_random is not None else "-"))
     out.append("\nReading: instruction issue is not what limits the loop (0.96 of peak with operands that do not toggle). With operands")
     out.append("that look like data the same instruction stream runs about 30 % slower: the switching activity costs power and the part")
     out.append("lowers its clock (the counter runs show about 2.0 GHz under the GEMMs against the 2.4 GHz of the data-sheet peak). The rate on")

@@ -107,3 +107,40 @@ def test_sweep_long_prints_its_rows(capsys):
         cells = [c.strip() for c in row.strip("|").split("|")]
         ms, std, T = float(cells[5]), float(cells[6]), int(cells[4])
         assert ms > 0 and std > 0 and abs(float(cells[8]) - T / ms * 1e3) <= 0.01 * T / ms * 1e3
+
+
+def test_profile_summary_cuts_encoder_steps_out_of_a_dispatch_sequence(tmp_path):
+    """The tables under profiles/ give every launch of a layer its own row: the seven layer kernels between an input
+    op and an output op, whatever else (table build, read-back copy, stand-alone loops) the trace holds."""
+    from effective_transformer_amd.sample import profile_summary as ps
+    layer = ["gemm_f16_pair_kernel<a>", "attention_kernel<b>", "gemm_f16_pair_kernel<a>", "bias_residual_layernorm_kernel<c>",
+             "gemm_f16_pair_kernel<d>", "gemm_f16_pair_kernel<a>", "bias_residual_layernorm_kernel<c>"]
+    step = ["scan_index_kernel", "compress_rows_kernel<x>", "seq_start_kernel", "seq_order_kernel",
+            "__amd_rocclr_copyBuffer"] + 2 * layer + ["restore_rows_kernel<x>"]
+    names = ["bias_gelu_kernel<h>"] * 3 + step + ["attention_kernel<b>"] * 4 + step + ["compress_rows_kernel<x>"] + layer
+    path = tmp_path / "t_kernel_trace.csv"
+    with open(path, "w") as f:
+        f.write("Kernel_Name,Start_Timestamp,End_Timestamp\n")
+        for i, n in enumerate(names):
+            f.write('"%s",%d,%d\n' % (n, 1000 * i, 1000 * i + 100 + i))
+    trace = ps.load_trace(str(path))
+    steps = ps.encoder_steps([t["kind"] for t in trace], layers=2)
+    assert len(steps) == 2 and all(len(b) == 14 for b in steps)          # the unfinished third step is left out
+    assert [names[i] for i in steps[0]] == 2 * layer
+    agg, short_names, n = ps.role_durations(trace, layers=2, skip=1)
+    assert n == 2 and set(agg) == set(ps.ROLES) and all(len(v) == 2 for v in agg.values())
+    first_qkv = steps[1][0]
+    assert agg["QKV"][0] == pytest.approx((100 + first_qkv) / 1e3)
+    assert ps.encoder_steps([t["kind"] for t in trace], layers=3) == []  # a different layer count matches nothing
+
+
+def test_profile_summary_prices_launches_with_the_documented_formulas():
+    from effective_transformer_amd.sample import profile_summary as ps
+    from effective_transformer_amd.sample.workloads import WORKLOADS
+    wl = WORKLOADS["cfg3"]
+    T, H, F, B, S, e = 40396, wl.H, wl.F, wl.B, wl.S, 2
+    assert ps.valid_tokens("cfg3") == T
+    a = ps.algorithmic("cfg3", T)
+    assert a["QKV"]["flops"] == 2.0 * T * 3 * H * H and a["FFN up + GELU"]["flops"] == 2.0 * T * F * H
+    assert a["attention"]["read"] + a["attention"]["write"] == 4 * T * H * e + B * S * S * e + 8 * T
+    assert a["LayerNorm 1"]["read"] + a["LayerNorm 1"]["write"] == 3 * T * H * e + 3 * H * e
