@@ -208,6 +208,8 @@ struct Entry {
 et_status dims_ok(et_handle h, int B, int S, int heads, int d) {
   ET_REQUIRE(h, B >= 1 && S >= 1 && heads >= 1 && d >= 1, "batch_size, seq_len, head_num, size_per_head must be >= 1");
   ET_REQUIRE(h, (long)B * S < (1L << 30), "batch_size * seq_len too large");
+  // row widths and their multiples (3 H, 4 H, bytes per row) are held in 32-bit integers throughout
+  ET_REQUIRE(h, (long)heads * d <= (1L << 20), "head_num * size_per_head above 1048576");
   return ET_OK;
 }
 
@@ -605,7 +607,7 @@ et_status et_output(et_handle h, et_dtype dtype, const void* from_tensor, const 
                     const int32_t* batch_idx, const int32_t* word_idx, void* to_tensor, int batch_size, int seq_len,
                     int head_num, int size_per_head, void* stream) {
   if (head_num < 1 || size_per_head < 1 || (long)head_num * size_per_head >= (1L << 30))
-    return fail(nullptr, ET_INVALID_ARGUMENT, "head_num, size_per_head must be >= 1");
+    return fail(h, ET_INVALID_ARGUMENT, "head_num, size_per_head must be >= 1");
   return et_restore(h, dtype, to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size, seq_len,
                     head_num * size_per_head, stream);
 }
@@ -620,7 +622,6 @@ et_status et_first_token(et_handle h, et_dtype dtype, const void* from_tensor, c
   if ((s = dims_ok(h, batch_size, seq_len, 1, hidden_dim)) != ET_OK) return s;
   ET_REQUIRE(h, from_tensor && to_tensor && valid_word_num_dev && batch_idx && word_idx, "null tensor pointer");
   const size_t row_bytes = (size_t)hidden_dim * et::elem_size(to_dt(dtype));
-  if (row_bytes % 16 != 0) return fail(h, ET_UNSUPPORTED, "hidden size in bytes must be a multiple of 16");
   et::launch_first_token(to_tensor, from_tensor, batch_idx, word_idx, valid_word_num_dev, batch_size * seq_len,
                          batch_size, (int)row_bytes, (hipStream_t)stream);
   return check_launch(h, "first token gather");

@@ -282,7 +282,8 @@ __global__ __launch_bounds__(1024) void seq_order_kernel(const int32_t* __restri
 // to[b,:] = row of the packed matrix that sits at position 0 of sequence b, zeros where sequence b has no token
 // there.  One wavefront per packed row (plus one past the end): the row that opens a sequence serves that sequence
 // and zeroes the token-less sequences in front of it, like seq_start_kernel walks the batch.
-__global__ __launch_bounds__(256) void first_token_kernel(u32x4* __restrict__ to, const u32x4* __restrict__ from,
+template <typename CH>
+__global__ __launch_bounds__(256) void first_token_kernel(CH* __restrict__ to, const CH* __restrict__ from,
                                                           const int32_t* __restrict__ batch_idx,
                                                           const int32_t* __restrict__ word_idx,
                                                           const int32_t* __restrict__ rows_dev, int rows_bound,
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(256) void first_token_kernel(u32x4* __restrict__ to
   const int prev = t == 0 ? -1 : min(batch_idx[t - 1], batch - 1);
   const int cur = t == T ? batch : min(batch_idx[t], batch - 1);
   if (cur == prev) return;                          // not the first row of its sequence
-  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const CH zero = {};
   for (int b = prev + 1; b < min(cur, batch); ++b)
     for (int c = lane; c < cpr; c += kWave) to[(size_t)b * cpr + c] = zero;
   if (t < T) {
@@ -309,8 +310,17 @@ void launch_first_token(void* to, const void* from, const int32_t* batch_idx, co
                         const int32_t* rows_dev, int rows_bound, int batch, int row_bytes, hipStream_t stream) {
   const int n = rows_bound + 1;
   const int per_wg = 256 / kWave;
-  first_token_kernel<<<(n + per_wg - 1) / per_wg, 256, 0, stream>>>((u32x4*)to, (const u32x4*)from, batch_idx, word_idx,
-                                                                    rows_dev, rows_bound, batch, row_bytes / 16);
+  const int grid = (n + per_wg - 1) / per_wg;
+  const int cb = row_bytes % 16 == 0 ? 16 : (row_bytes % 4 == 0 ? 4 : 2);      // as the row movers below
+  if (cb == 16)
+    first_token_kernel<u32x4><<<grid, 256, 0, stream>>>((u32x4*)to, (const u32x4*)from, batch_idx, word_idx, rows_dev,
+                                                        rows_bound, batch, row_bytes / 16);
+  else if (cb == 4)
+    first_token_kernel<uint32_t><<<grid, 256, 0, stream>>>((uint32_t*)to, (const uint32_t*)from, batch_idx, word_idx,
+                                                           rows_dev, rows_bound, batch, row_bytes / 4);
+  else
+    first_token_kernel<uint16_t><<<grid, 256, 0, stream>>>((uint16_t*)to, (const uint16_t*)from, batch_idx, word_idx,
+                                                           rows_dev, rows_bound, batch, row_bytes / 2);
 }
 
 size_t scan_scratch_words(int length) {

@@ -127,7 +127,7 @@ et_status et_input_static(et_handle h, et_dtype dtype, const void* from_tensor, 
  * layer, :99-101).
  * from_seq_len must equal to_seq_len (tf_op/bert_transformer_op.cc:130-131).  `out` must not
  * alias from_tensor/to_tensor.  Shapes: seq_len <= 1024, batch_size <= 65535, any size_per_head from 1 to 256 (see
- * et_attention).  The tuned kernels take head size 64 and hidden sizes in multiples of 32 (fp16) or 16 (fp32); every
+ * et_attention), head_num * size_per_head <= 1048576 (every entry point), activations below 4 GB per matrix.  The tuned kernels take head size 64 and hidden sizes in multiples of 32 (fp16) or 16 (fp32); every
  * other shape runs element-wise kernels with the same arithmetic (the reference's kernels index by element too,
  * cuda/attention.cu:190-219). */
 et_status et_layer(et_handle h, et_dtype dtype, const et_layer_weights* weights,

@@ -161,3 +161,6 @@ def test_input_and_output_ops_with_odd_rows(dtype, H):
     back = ops.effective_transformer_output(to, vwn, bidx, widx, B, S, S, 1, H).cpu().numpy()
     want = np.where(mask[:, :, None].astype(bool), x, 0).astype(x.dtype)
     assert np.array_equal(back.view(np.uint8), want.view(np.uint8))
+    # the first-token gather moves rows in the same pieces
+    first = ops.effective_transformer_first_token(to, vwn, bidx, widx).cpu().numpy()
+    assert np.array_equal(first.view(np.uint8), want[:, 0, :].view(np.uint8))
