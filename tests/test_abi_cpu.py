@@ -71,3 +71,31 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0
     assert "ONE GPU" in (r.stderr + r.stdout)
     assert "{" not in r.stdout
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """include/et.h is what a C (or cgo / JNI) caller includes: it must compile as strict C99, and a C program must link
+    against the library and get sizes and status strings without a GPU."""
+    import shutil
+    import subprocess
+    from effective_transformer_amd import _lib
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "caller.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "et.h"\n'
+        "int main(void) {\n"
+        "  et_layer_weights w; et_layer_prepared p; memset(&w, 0, sizeof w); memset(&p, 0, sizeof p);\n"
+        "  if (et_layer_workspace_bytes(ET_FP16, 8, 32, 12, 64) == 0 || et_seq_workspace_bytes(8) < (2 * 8 + 1) * 4) return 1;\n"
+        '  if (strcmp(et_status_string(ET_WORKSPACE_TOO_SMALL), "ET_WORKSPACE_TOO_SMALL") != 0) return 2;\n'
+        "  if (et_output(NULL, ET_FP16, NULL, NULL, NULL, NULL, NULL, 1, 1, 1, 1, NULL) != ET_INVALID_ARGUMENT) return 3;\n"
+        '  printf("%s\\n", et_last_error(NULL));\n'
+        "  return 0;\n}\n")
+    exe = tmp_path / "caller"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    inc = os.path.join(os.path.dirname(os.path.dirname(libdir)), "include")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, str(src), "-o", str(exe),
+                    "-L", libdir, "-let_hip", "-Wl,-rpath," + libdir], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    assert "null handle" in r.stdout
