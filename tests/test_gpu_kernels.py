@@ -376,6 +376,67 @@ def test_fused_attention_long_sequences_same_bits_in_any_batch(k, dtype, S):
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+@pytest.mark.parametrize("S", [40, 64, 100, 128])
+@pytest.mark.parametrize("layout", [1, 0])
+def test_fused_attention_mixed_lengths_same_bits_in_any_batch(k, dtype, S, layout):
+    """The kernel for up to 128 positions on a batch of very different sequences: every sequence must give the bits it
+    gives alone in a batch of one, whatever stands beside it, and match the oracle: short and long sequences,
+    token-less ones, a short one whose tokens sit at late positions, holes, and masks that attend to padded keys
+    (their zero scores count in the softmax of the sequence they belong to)."""
+    print("attention mixed lengths", dtype, S, layout, flush=True)
+    heads, d = 4, 64
+    H = heads * d
+    rng = np.random.RandomState(S + layout)
+    half = 32 if S <= 64 else 64
+    masks = []
+    for n in [1, 5, half, half - 1, half + 1, S, 0, 17, 3, S - 2, 9, half, 2, 30, 0, 12, 7]:
+        m = np.zeros(S, np.int32)
+        m[:min(n, S)] = 1
+        masks.append(m)
+    late = np.zeros(S, np.int32); late[[0, S // 2 + 3, S - 1]] = 1                # three tokens, the last position in use
+    holes = np.zeros(S, np.int32); holes[[1, 4, 5, half - 1]] = 1                  # fits a half
+    holes2 = (rng.random_sample(S) < 0.3).astype(np.int32); holes2[half:] = 0      # fits a half
+    masks += [late, holes, holes2]
+    n_seq = len(masks)
+    lens = [int(m.sum()) for m in masks]
+    rows = [o.rnd(rng.randn(n, 3 * H), dtype) for n in lens]
+    attr_seq = [o.rnd((rng.random_sample((S, S)) < 0.7).astype(np.float32), dtype) for _ in masks]
+
+    def run(order):
+        B = len(order)
+        mask = np.stack([masks[j] for j in order])
+        _, T, bi, wi, _ = o.input_op_fast(np.zeros((B, S, 1), np.float32), mask)
+        packed = np.zeros((B * S, 3 * H), o._np_dtype(dtype))
+        if T:
+            packed[:T] = np.concatenate([rows[j] for j in order])
+        attr = np.stack([attr_seq[j] for j in order])
+        p = dict(B=B, S=S, T=T, bi=bi, wi=wi)
+        bi_d, wi_d, vwn = _idx_dev(p)
+        z = np.zeros(H, o._np_dtype(dtype))
+        qp, kp, vp = o.add_qkv_bias_padding(packed[:T, :H], z, packed[:T, H:2 * H], z, packed[:T, 2 * H:], z, T, B, S, heads,
+                                            d, bi, wi, dtype)
+        if layout == 1:
+            pk = dev(packed)
+            out = k.attention(pk, pk[:, H:], pk[:, 2 * H:], 1, 3 * H, dev(attr), vwn, B, S, heads, d, bi_d, wi_d).cpu().numpy()
+        else:
+            out = k.attention(dev(qp), dev(kp), dev(vp), 0, 0, dev(attr), vwn, B, S, heads, d, bi_d, wi_d).cpu().numpy()
+        want = o.attention(qp, kp, vp, attr, T, bi, wi, dtype)
+        if dtype == "fp32":
+            np.testing.assert_allclose(out[:T], want, rtol=1e-4, atol=2e-5)
+        else:
+            np.testing.assert_allclose(out[:T].astype(np.float32), want.astype(np.float32), rtol=4e-3, atol=4e-3)
+        starts = np.concatenate([[0], np.cumsum([lens[j] for j in order])])
+        return {j: out[starts[i]:starts[i + 1]] for i, j in enumerate(order)}
+
+    a = run(list(range(n_seq)))
+    b = run(list(rng.permutation(n_seq)))
+    for j in range(n_seq):
+        assert np.array_equal(a[j], b[j]), j
+    for j in [0, 2, 4, 5, n_seq - 3, n_seq - 2, n_seq - 1]:
+        assert np.array_equal(a[j], run([j])[j]), j
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
 def test_fused_attention_many_sequences_head_groups(k, dtype):
     """A batch large enough that one workgroup serves a group of 4 heads (shared mask registers, positions and
     zero fill across heads, next head prefetched): holes in the mask, an attention mask unrelated to it."""
