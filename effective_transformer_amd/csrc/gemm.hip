@@ -541,6 +541,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_persistent_kernel(GemmArgs
 constexpr int kQAPair = kPBM * 128;                            // 32 KB: 256 rows x two k-steps
 constexpr int kQPair = kQAPair + kPBN * 128;                   // 64 KB: A rows, then B^T rows
 constexpr int kQSmem = 2 * kQPair;
+constexpr int kQSmemA3 = 3 * kQAPair + 2 * (kQPair - kQAPair);   // 160 KB: three A slots, two B^T slots
 
 __device__ __forceinline__ int pair_swizzle(int row) { return (row >> 1) & 7; }
 
@@ -550,7 +551,11 @@ __device__ __forceinline__ int pair_swizzle(int row) { return (row >> 1) & 7; }
 // descriptor and cost no traffic.
 // NT: C leaves through non-temporal stores (a matrix too big to be found in the last-level cache by its reader);
 // plain stores otherwise.
-template <bool GELU, int MI, bool NT>
+// A3: three LDS slots for A instead of two, all of the 160 KB: the A rows of a pair are requested three pairs ahead
+// of their first use instead of two (B^T as before).  For the projection whose A is the big matrix and comes from
+// HBM (k >= 2048: FFN-down), where a pair's time does not cover that latency.  Same instructions on the same data in
+// the same order: same bits.
+template <bool GELU, int MI, bool NT, bool A3 = false>
 __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only types in the body; the host pass only needs the stub
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -630,22 +635,37 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
     voff_b[j] = ((uint32_t)col * (uint32_t)K + (uint32_t)c * 8u) * 2u;
   }
   const int a_pair_bytes = args.a_blocked ? kQAPair : 128;       // from one pair of k-steps of A to the next
-  // instruction q (0..3: A, 4..7: B^T) of this wave's share of pair `pr` of a tile into slot `slot`
-  auto issue1 = [&](int slot, int pr, const __amdgpu_buffer_rsrc_t& ra, const __amdgpu_buffer_rsrc_t& rb, int q) {
-    unsigned char* st = smem + slot * kQPair;
-    if (q < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, ET_LDS_PTR(st + (wave * 4 + q) * 1024), 16, voff_a[q],
-                                               pr * a_pair_bytes, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, ET_LDS_PTR(st + kQAPair + (wave * 4 + q - 4) * 1024), 16,
-                                               voff_b[q - 4], pr * 128, 0, 0);
+  // LDS: slot s = A rows, then B^T rows of a pair (two slots); with A3 a ring of three A slots, then two B^T slots
+  auto a_slot = [&](int sa) -> unsigned char* { return smem + sa * (A3 ? kQAPair : kQPair); };
+  auto b_slot = [&](int sb) -> unsigned char* {
+    return A3 ? smem + 3 * kQAPair + sb * (kQPair - kQAPair) : smem + sb * kQPair + kQAPair;
+  };
+  // instruction q (0..3) of this wave's share of the A rows / B^T rows of pair `pr` of a tile into slot sa / sb
+  auto issue_a = [&](int sa, int pr, const __amdgpu_buffer_rsrc_t& ra, int q) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, ET_LDS_PTR(a_slot(sa) + (wave * 4 + q) * 1024), 16, voff_a[q],
+                                             pr * a_pair_bytes, 0, 0);
+  };
+  auto issue_b = [&](int sb, int pr, const __amdgpu_buffer_rsrc_t& rb, int q) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, ET_LDS_PTR(b_slot(sb) + (wave * 4 + q) * 1024), 16, voff_b[q], pr * 128,
+                                             0, 0);
+  };
+  // instruction q (0..7) of a whole pair: A first, then B^T; with A3 the other way round, and the A rows are those
+  // of the pair one further ahead, so that they are the newest requests and may stay in flight at the next wait
+  auto issue1 = [&](int sa, int sb, int pr_a, int pr_b, const __amdgpu_buffer_rsrc_t& ra,
+                    const __amdgpu_buffer_rsrc_t& rb, int q) {
+    if (A3) {
+      if (q < 4) issue_b(sb, pr_b, rb, q);
+      else issue_a(sa, pr_a, ra, q - 4);
+    } else {
+      if (q < 4) issue_a(sa, pr_a, ra, q);
+      else issue_b(sb, pr_b, rb, q - 4);
+    }
   };
 
   // operand reads: row (wm*128 + i*16 + l16) resp. (wn*64 + j*16 + l16), chunk (4*half + g), swizzled
   const int sw = pair_swizzle(l16);
   const int a_rd[2] = {(wm * 16 * MI + l16) * 128 + ((g ^ sw) * 16), (wm * 16 * MI + l16) * 128 + (((4 + g) ^ sw) * 16)};
-  const int b_rd[2] = {kQAPair + (wn * 64 + l16) * 128 + ((g ^ sw) * 16),
-                       kQAPair + (wn * 64 + l16) * 128 + (((4 + g) ^ sw) * 16)};
+  const int b_rd[2] = {(wn * 64 + l16) * 128 + ((g ^ sw) * 16), (wn * 64 + l16) * 128 + (((4 + g) ^ sw) * 16)};
 
   int idx = local;
   if (!valid(idx)) return;
@@ -668,22 +688,24 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
   half8 a[2][MI], b[2][4];
   int pairs_done = 0;                            // by this workgroup: slot of a pair = pairs_done & 1
 
-  // One k-step: MFMAs on operand set P; half `rh` of slot `rs` is read into the other set; with DMA set, this wave's
-  // eight DMA instructions for pair `dpr` (descriptors da, db) go into slot `ds`, one after each group of four MFMAs.
-  auto step = [&](auto Pc, auto FIRSTc, auto DMAc, int rs, int ds, int dpr, const __amdgpu_buffer_rsrc_t& da,
-                  const __amdgpu_buffer_rsrc_t& db) {
+  // One k-step: MFMAs on operand set P; half `rh` of the slots rsa / rsb is read into the other set; with DMA set, this
+  // wave's eight DMA instructions (A rows of pair dpa into slot dsa, B^T rows of pair dpb into slot dsb; descriptors
+  // da, db) go out, one after each group of four MFMAs.
+  auto step = [&](auto Pc, auto FIRSTc, auto DMAc, int rsa, int rsb, int dsa, int dsb, int dpa, int dpb,
+                  const __amdgpu_buffer_rsrc_t& da, const __amdgpu_buffer_rsrc_t& db) {
     constexpr int P = decltype(Pc)::value;
     constexpr bool FIRST = decltype(FIRSTc)::value;
     constexpr bool DMA = decltype(DMAc)::value;
     constexpr int rh = 1 - P;                    // the even step reads half 1 of its own pair, the odd step half 0 of the next
-    const unsigned char* ns = smem + rs * kQPair;
+    const unsigned char* nsa = a_slot(rsa);
+    const unsigned char* nsb = b_slot(rsb);
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       // two of the 4 + MI operand reads of the next step in front of each group of four MFMAs (B^T blocks first)
 #pragma unroll
       for (int r = 2 * i; r < 2 * i + 2 && r < 4 + MI; ++r) {
-        if (r < 4) b[1 - P][r] = *reinterpret_cast<const half8*>(ns + b_rd[rh] + r * 2048);
-        else a[1 - P][r - 4] = *reinterpret_cast<const half8*>(ns + a_rd[rh] + (r - 4) * 2048);
+        if (r < 4) b[1 - P][r] = *reinterpret_cast<const half8*>(nsb + b_rd[rh] + r * 2048);
+        else a[1 - P][r - 4] = *reinterpret_cast<const half8*>(nsa + a_rd[rh] + (r - 4) * 2048);
       }
       // the column blocks back and forth: between two MFMAs only one operand changes, which costs measurably less
       // power than the row-major order (the part runs the same stream 1 - 2 % faster on random operands)
@@ -696,7 +718,7 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
       if (DMA) {
 #pragma unroll
         for (int q = 0; q < 8; ++q)
-          if (q * MI / 8 == i) issue1(ds, dpr, da, db, q);      // the eight DMA instructions spread over the MI groups
+          if (q * MI / 8 == i) issue1(dsa, dsb, dpa, dpb, da, db, q);      // the eight DMA instructions spread over the MI groups
       }
       __builtin_amdgcn_sched_barrier(0);         // keeps the reads and the DMA where they are between the MFMA groups
     }
@@ -704,17 +726,29 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
   using Even = std::integral_constant<int, 0>;
   using Odd = std::integral_constant<int, 1>;
 
-  // pairs 0 and 1 of the first tile, operands of k-step 0
+  // pairs 0 and 1 of the first tile (with A3 also the A rows of pair 2), operands of k-step 0
 #pragma unroll
-  for (int q = 0; q < 8; ++q) issue1(0, 0, cur.a, cur.b, q);
+  for (int q = 0; q < 4; ++q) issue_a(0, 0, cur.a, q);
 #pragma unroll
-  for (int q = 0; q < 8; ++q) issue1(1, 1, cur.a, cur.b, q);
-  wait_vmcnt<8>();
+  for (int q = 0; q < 4; ++q) issue_b(0, 0, cur.b, q);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) issue_a(1, 1, cur.a, q);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) issue_b(1, 1, cur.b, q);
+  if (A3) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) issue_a(2, 2, cur.a, q);
+    wait_vmcnt<12>();
+  } else {
+    wait_vmcnt<8>();
+  }
   barrier_only();
 #pragma unroll
-  for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const half8*>(smem + b_rd[0] + j * 2048);
+  for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const half8*>(b_slot(0) + b_rd[0] + j * 2048);
 #pragma unroll
-  for (int i = 0; i < MI; ++i) a[0][i] = *reinterpret_cast<const half8*>(smem + a_rd[0] + i * 2048);
+  for (int i = 0; i < MI; ++i) a[0][i] = *reinterpret_cast<const half8*>(a_slot(0) + a_rd[0] + i * 2048);
+  int sa = 0;                                    // A slot of the current pair = pairs_done % 3 (A3)
+  auto next3 = [](int v) { return v == 2 ? 0 : v + 1; };
 
   bool first_tile = true;
   while (true) {
@@ -726,32 +760,45 @@ __global__ __launch_bounds__(kPThreads) void gemm_f16_pair_kernel(GemmArgs args)
     if (computes) {
       for (int p = 0; p < np; ++p) {
         const int s = pairs_done & 1;
-        if (p == 0) step(Even{}, std::true_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
-        else step(Even{}, std::false_type{}, std::false_type{}, s, 0, 0, cur.a, cur.b);
+        const int ra = A3 ? sa : s;                // this pair's A slot
+        if (p == 0) step(Even{}, std::true_type{}, std::false_type{}, ra, s, 0, 0, 0, 0, cur.a, cur.b);
+        else step(Even{}, std::false_type{}, std::false_type{}, ra, s, 0, 0, 0, 0, cur.a, cur.b);
         // this wave's share of the next pair has landed (right after a tile boundary that was confirmed before the C
-        // stores went out) and its last reads of slot s, which feed the odd step, are complete
-        if (first_tile || p >= 1) wait_vmcnt<0>();
+        // stores went out) and its last reads of slot s, which feed the odd step, are complete; with A3 the four
+        // newest requests, the A rows of the pair after the next, may still be on their way
+        if (first_tile || p >= 1) {
+          if (A3) wait_vmcnt<4>();
+          else wait_vmcnt<0>();
+        }
         wait_lgkmcnt0();
         barrier_only();
-        // pair p+2 of this tile, or the matching pair of the next one, replaces slot s
-        const bool in_tile = p + 2 < np;
-        const __amdgpu_buffer_rsrc_t da = in_tile ? cur.a : nxt.a;
-        const __amdgpu_buffer_rsrc_t db = in_tile ? cur.b : nxt.b;
-        step(Odd{}, std::false_type{}, std::true_type{}, s ^ 1, s, in_tile ? p + 2 : p + 2 - np, da, db);
+        // B^T of pair p+2 (A of pair p+2, with A3 of pair p+3) of this tile, or the matching pair of the next one,
+        // replaces what this pair held
+        const int pa = A3 ? p + 3 : p + 2, pb = p + 2;
+        const __amdgpu_buffer_rsrc_t da = pa < np ? cur.a : nxt.a;
+        const __amdgpu_buffer_rsrc_t db = pb < np ? cur.b : nxt.b;
+        step(Odd{}, std::false_type{}, std::true_type{}, A3 ? next3(sa) : s ^ 1, s ^ 1, ra, s, pa < np ? pa : pa - np,
+             pb < np ? pb : pb - np, da, db);
         ++pairs_done;
+        sa = next3(sa);
       }
     } else {
       // the other half's waves: same barriers, same share of the DMA, no operand reads and no MFMAs
       for (int p = 0; p < np; ++p) {
         const int s = pairs_done & 1;
-        if (first_tile || p >= 1) wait_vmcnt<0>();
+        if (first_tile || p >= 1) {
+          if (A3) wait_vmcnt<4>();
+          else wait_vmcnt<0>();
+        }
         barrier_only();
-        const bool in_tile = p + 2 < np;
-        const __amdgpu_buffer_rsrc_t da = in_tile ? cur.a : nxt.a;
-        const __amdgpu_buffer_rsrc_t db = in_tile ? cur.b : nxt.b;
+        const int pa = A3 ? p + 3 : p + 2, pb = p + 2;
+        const __amdgpu_buffer_rsrc_t da = pa < np ? cur.a : nxt.a;
+        const __amdgpu_buffer_rsrc_t db = pb < np ? cur.b : nxt.b;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) issue1(s, in_tile ? p + 2 : p + 2 - np, da, db, q);
+        for (int q = 0; q < 8; ++q)
+          issue1(A3 ? sa : s, s, pa < np ? pa : pa - np, pb < np ? pb : pb - np, da, db, q);
         ++pairs_done;
+        sa = next3(sa);
       }
     }
     wait_vmcnt<0>();
@@ -1235,11 +1282,12 @@ int pair_kernel_row_blocks(int m_bound, int n, int groups) {
   return best_mi;
 }
 
-template <bool GELU, int MI, bool NT>
+template <bool GELU, int MI, bool NT, bool A3 = false>
 void launch_pair(const GemmArgs& a, int grid, hipStream_t stream) {
-  auto kern = gemm_f16_pair_kernel<GELU, MI, NT>;
-  allow_dynamic_lds(reinterpret_cast<const void*>(kern), kQSmem);
-  kern<<<grid, kPThreads, kQSmem, stream>>>(a);
+  auto kern = gemm_f16_pair_kernel<GELU, MI, NT, A3>;
+  constexpr int lds = A3 ? kQSmemA3 : kQSmem;
+  allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
+  kern<<<grid, kPThreads, lds, stream>>>(a);
 }
 
 void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
@@ -1275,6 +1323,14 @@ void launch_f16_persistent(GemmArgs a, hipStream_t stream, bool b_transposed) {
   if (!b_transposed) {
     allow_dynamic_lds(reinterpret_cast<const void*>(gemm_f16_persistent_kernel), kPSmem);
     gemm_f16_persistent_kernel<<<grid, kPThreads, kPSmem, stream>>>(a);
+    return;
+  }
+  // A from HBM, few long tiles per workgroup: the A rows are requested a pair earlier (three LDS slots for A)
+  if (!a.gelu && a.k >= 2048 && mi >= 7) {
+    if (mi == 8 && !a.c_cached) launch_pair<false, 8, true, true>(a, grid, stream);
+    else if (mi == 8) launch_pair<false, 8, false, true>(a, grid, stream);
+    else if (!a.c_cached) launch_pair<false, 7, true, true>(a, grid, stream);
+    else launch_pair<false, 7, false, true>(a, grid, stream);
     return;
   }
 #define ET_PAIR_CASE(M)                                                      \
